@@ -1,0 +1,149 @@
+/*
+ * we_attn.h - C ABI of the MI355X (gfx950) frame-causal ring-buffer attention library.
+ *
+ * The library replaces, for one DiT attention layer and one frame, the work world_engine
+ * does between its q/k/v projection and its output projection:
+ *
+ *   RoPE(q), RoPE(k)                      src/model/attn.py:22-40, :110
+ *   kv_cache.upsert(k, v, pos_ids, layer) src/model/kv_cache.py:104-154, :191-193
+ *   flex_attention(q, k, v, block_mask)   src/model/attn.py:116, src/patch_model.py:133
+ *
+ * world_engine has no native code: these are the calls a binding would replace with the two
+ * entry points below.  All pointers are DEVICE pointers owned by the caller.  Every call only
+ * enqueues work on `stream`; it never synchronises, never allocates and keeps no mutable
+ * global state (beyond raising each kernel's dynamic-LDS limit once), so it is re-entrant and
+ * capturable into a HIP graph.  The frame index that
+ * selects the ring slot is read by the kernels from device memory (`t_pos[0]`), exactly as the
+ * reference derives it from a device tensor (src/model/kv_cache.py:126), so no host value of
+ * it is ever needed.
+ *
+ * Return value: 0 on success, a negative WE_ERR_* code otherwise (nothing is launched then).
+ */
+#ifndef WE_ATTN_H
+#define WE_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types of q/k/v, the cache buffer and the attention output */
+#define WE_DTYPE_BF16 0
+#define WE_DTYPE_F16 1
+#define WE_DTYPE_F32 2 /* we_rope_kv_store only */
+
+#define WE_OK 0
+#define WE_ERR_NULL_POINTER (-1)
+#define WE_ERR_BAD_SHAPE (-2)     /* zero/negative sizes, L % T != 0, (L/T) % dilation != 0, H % Hkv != 0 */
+#define WE_ERR_UNSUPPORTED (-3)   /* head dim, frame length, slot count or dtype outside what the kernels cover */
+#define WE_ERR_ALIGNMENT (-4)     /* pointer or stride not 16-byte aligned */
+#define WE_ERR_WORKSPACE (-5)     /* split-context workspace missing or too small */
+#define WE_ERR_LAUNCH (-6)        /* the HIP runtime refused the launch */
+
+#define WE_MAX_SLOTS 256 /* maximum number of ring slots L / T */
+
+/* Library version: major*10000 + minor*100 + patch. */
+int we_version(void);
+
+/* Static description of a WE_ERR_* code. */
+const char* we_error_string(int code);
+
+/*
+ * Fused RoPE + ring-slot K/V store for one frame.
+ *
+ * Replaces RoPE.forward on q and k (src/model/attn.py:33-40), torch.stack([k, v])
+ * (src/model/kv_cache.py:192), the tail index_copy_ (:138), the unfrozen ring index_copy_ and
+ * the `written` update (:147-151), with the slot arithmetic of :126-131,:140 done on the device.
+ *
+ *   q        [B, H,   T, Dh]  element strides q_strides  = {batch, head, token}; Dh contiguous.
+ *                             May be NULL (then q_out must be NULL): K/V store only.
+ *   k, v     [B, Hkv, T, Dh]  element strides k_strides / v_strides, same convention.
+ *   q_out    [B, H, T, Dh] contiguous: RoPE(q).
+ *   cos_table, sin_table  [table_rows, Dh/2] fp32.  Both NULL: no rotation (k is stored as
+ *            given, q is copied), which is the behaviour of StaticKVCache.upsert on an already
+ *            rotated k.
+ *   t_pos, y_pos, x_pos   int64 [B, T], row stride pos_stride_b.  Table row of token (b, i) is
+ *            t_pos*grid_h*grid_w + y_pos*grid_w + x_pos (src/model/attn.py:27), clamped into
+ *            [0, table_rows).  y_pos/x_pos may be NULL when the tables are NULL.
+ *            t_pos[0] is the frame index that selects the ring slot.
+ *   kv       [2, B, Hkv, L + T, Dh] contiguous cache buffer (plane 0 = K, 1 = V).
+ *   written  [L + T] bytes (torch.bool).
+ *   L        ring length in tokens (multiple of T); dilation = pinned_dilation, divides L/T.
+ *   is_frozen  non-zero: only the tail rows [L, L+T) are written.  Zero: additionally, when
+ *            t_pos[0] % dilation == 0, rows [slot*T, (slot+1)*T) with
+ *            slot = ceil(t_pos[0]/dilation) % ((L/T)/dilation) are written and marked in
+ *            `written`; otherwise the tail is marked.
+ *
+ * Rotation is computed in fp32 with separately rounded products and rounded once to the
+ * element type (round-to-nearest-even), so ring contents are bit-identical to eager PyTorch.
+ * Requirements: Dh % 16 == 0; all pointers and row starts 16-byte aligned.
+ */
+int we_rope_kv_store(const void* q, const void* k, const void* v,
+                     const int64_t q_strides[3], const int64_t k_strides[3],
+                     const int64_t v_strides[3], void* q_out,
+                     const float* cos_table, const float* sin_table, int64_t table_rows,
+                     const int64_t* t_pos, const int64_t* y_pos, const int64_t* x_pos,
+                     int64_t pos_stride_b, int64_t grid_h, int64_t grid_w,
+                     void* kv, uint8_t* written,
+                     int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L,
+                     int32_t dilation, int32_t is_frozen, int32_t dtype, void* stream);
+
+/*
+ * RoPE alone on one [B, H, T, Dh] tensor: x_out = RoPE(x), x_out contiguous.  Replaces a
+ * stand-alone RoPE.forward call (src/model/attn.py:33-40); same arithmetic, arguments and
+ * requirements as the rotation inside we_rope_kv_store.
+ */
+int we_rope_apply(const void* x, const int64_t x_strides[3], void* x_out,
+                  const float* cos_table, const float* sin_table, int64_t table_rows,
+                  const int64_t* t_pos, const int64_t* y_pos, const int64_t* x_pos,
+                  int64_t pos_stride_b, int64_t grid_h, int64_t grid_w,
+                  int32_t B, int32_t H, int32_t T, int32_t Dh, int32_t dtype, void* stream);
+
+/*
+ * Number of context splits we_attn_ring_fwd picks when called with n_splits = 0.
+ */
+int32_t we_attn_auto_splits(int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L);
+
+/*
+ * Bytes of workspace we_attn_ring_fwd needs for a given split count (0 when n_splits <= 1).
+ */
+size_t we_attn_workspace_bytes(int32_t B, int32_t H, int32_t T, int32_t Dh, int32_t n_splits);
+
+/*
+ * Frame-block-causal attention of one frame's queries over the ring buffer.
+ *
+ * Replaces make_block_mask (src/model/kv_cache.py:12-61, :141-144) and the flex_attention call
+ * (src/model/attn.py:116).  Key row j of the cache is visible iff it lies in the tail
+ * [L, L+T), or in a ring slot s with written[s*T] != 0 that is not the slot the current frame
+ * maps to on a persisting frame (t_pos[0] % dilation == 0).  Visibility does not depend on
+ * batch, head or query, so no mask tensor is materialised: the kernel walks the visible slots
+ * of `kv` in place.  out = softmax(scale * q k^T) v over the visible keys, fp32 accumulation,
+ * probabilities rounded to the element type before the second product.
+ *
+ *   q    [B, H, T, Dh]   element strides q_strides = {batch, head, token}; Dh contiguous.
+ *   kv, written, t_pos   as in we_rope_kv_store, after that call for the same frame.
+ *   out  [B, H, T, Dh]   element strides out_strides = {batch, head, token}; Dh contiguous.
+ *   workspace            device scratch of at least we_attn_workspace_bytes(..., n_splits)
+ *                        bytes when the effective split count is > 1; may be NULL otherwise.
+ *   n_splits             0 = choose automatically; 1 = single pass; 2..64 = split the visible
+ *                        context into that many parts and combine them in a second kernel.
+ *   q_tile               queries per workgroup: 0 = choose automatically, or 128 / 256.
+ *   scale                softmax scale (> 0); the reference uses 1/sqrt(Dh).
+ *
+ * Requirements: dtype bf16 or f16; Dh in {64, 128}; T % 64 == 0; L/T <= WE_MAX_SLOTS;
+ * H % Hkv == 0; pointers and row starts 16-byte aligned.
+ */
+int we_attn_ring_fwd(const void* q, const int64_t q_strides[3],
+                     const void* kv, const uint8_t* written, const int64_t* t_pos,
+                     void* out, const int64_t out_strides[3],
+                     void* workspace, size_t workspace_bytes,
+                     int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L,
+                     int32_t dilation, float scale, int32_t n_splits, int32_t q_tile,
+                     int32_t dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* WE_ATTN_H */

@@ -1,0 +1,156 @@
+"""CPU-side checks: the C-ABI library loads and exports every declared symbol, argument
+validation returns the documented codes before anything touches a GPU, and the host classes
+mirror the reference's interface."""
+import ctypes
+import os
+import re
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+import world_engine_amd as wea
+from world_engine_amd import _capi, ops
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "we_attn.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(we_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_symbols()
+    assert {"we_version", "we_error_string", "we_rope_kv_store", "we_rope_apply", "we_attn_auto_splits",
+            "we_attn_workspace_bytes", "we_attn_ring_fwd"} <= set(names)
+    assert set(names) == set(_capi.SIGNATURES), "ctypes signatures and header disagree"
+    lib = _capi.lib()
+    for n in names:
+        assert hasattr(lib, n), f"{n} not exported"
+    assert lib.we_version() >= 100
+    assert lib.we_error_string(0) == b"ok" and b"unknown" in lib.we_error_string(-99)
+
+
+def test_validation_codes_without_gpu():
+    lib = _capi.lib()
+    s3 = _capi.i64x3(8, 8, 8)
+    fake = ctypes.c_void_p(4096)     # never dereferenced: validation fails first
+    # null pointers
+    assert lib.we_attn_ring_fwd(None, s3, fake, fake, fake, fake, s3, None, 0, 1, 1, 1, 64, 64, 64, 1, 0.1, 1, 0, 0, None) == -1
+    # L not a multiple of T
+    assert lib.we_attn_ring_fwd(fake, s3, fake, fake, fake, fake, s3, None, 0, 1, 1, 1, 64, 64, 100, 1, 0.1, 1, 0, 0, None) == -2
+    # H % Hkv != 0
+    assert lib.we_attn_ring_fwd(fake, s3, fake, fake, fake, fake, s3, None, 0, 1, 3, 2, 64, 64, 64, 1, 0.1, 1, 0, 0, None) == -2
+    # unsupported head dim / frame length / dtype / slot count
+    assert lib.we_attn_ring_fwd(fake, s3, fake, fake, fake, fake, s3, None, 0, 1, 1, 1, 64, 96, 64, 1, 0.1, 1, 0, 0, None) == -3
+    assert lib.we_attn_ring_fwd(fake, s3, fake, fake, fake, fake, s3, None, 0, 1, 1, 1, 48, 64, 96, 1, 0.1, 1, 0, 0, None) == -3
+    assert lib.we_attn_ring_fwd(fake, s3, fake, fake, fake, fake, s3, None, 0, 1, 1, 1, 64, 64, 64, 1, 0.1, 1, 0, 2, None) == -3
+    assert lib.we_attn_ring_fwd(fake, s3, fake, fake, fake, fake, s3, None, 0, 1, 1, 1, 64, 64, 64 * 257, 1, 0.1, 1, 0, 0, None) == -3
+    # misaligned pointer / stride
+    assert lib.we_attn_ring_fwd(ctypes.c_void_p(4100), s3, fake, fake, fake, fake, s3, None, 0, 1, 1, 1, 64, 64, 64, 1, 0.1, 1, 0, 0, None) == -4
+    assert lib.we_attn_ring_fwd(fake, _capi.i64x3(8, 8, 4), fake, fake, fake, fake, s3, None, 0, 1, 1, 1, 64, 64, 64, 1, 0.1, 1, 0, 0, None) == -4
+    # splits without workspace
+    assert lib.we_attn_ring_fwd(fake, s3, fake, fake, fake, fake, s3, None, 0, 1, 1, 1, 64, 64, 64, 1, 0.1, 2, 0, 0, None) == -5
+    # store: q without q_out, tables without y/x, dilation not dividing the slot count
+    assert lib.we_rope_kv_store(fake, fake, fake, s3, s3, s3, None, None, None, 0, fake, None, None, 0, 1, 1, fake, fake,
+                                1, 1, 1, 64, 64, 64, 1, 0, 0, None) == -1
+    assert lib.we_rope_kv_store(None, fake, fake, None, s3, s3, None, fake, fake, 10, fake, None, None, 0, 1, 1, fake, fake,
+                                1, 1, 1, 64, 64, 64, 1, 0, 0, None) == -1
+    assert lib.we_rope_kv_store(None, fake, fake, None, s3, s3, None, None, None, 0, fake, None, None, 0, 1, 1, fake, fake,
+                                1, 1, 1, 64, 64, 192, 2, 0, 0, None) == -2
+
+
+def test_workspace_and_split_planning():
+    lib = _capi.lib()
+    assert lib.we_attn_workspace_bytes(1, 16, 256, 128, 1) == 0
+    assert lib.we_attn_workspace_bytes(1, 16, 256, 128, 4) == 4 * 16 * 256 * (128 + 2) * 4
+    # 256-token frames need context splits to fill the chip, 1024-token frames with 96 heads do not
+    assert lib.we_attn_auto_splits(1, 16, 16, 256, 128, 4096) > 1
+    assert lib.we_attn_auto_splits(4, 24, 24, 1024, 128, 8192) == 1
+    # never more splits than half the 64-key tiles of the context
+    assert lib.we_attn_auto_splits(1, 1, 1, 64, 64, 128) <= 1
+
+
+def test_no_cpu_fallback():
+    cache = wea.LayerKVCache(1, 2, 128, 64, torch.bfloat16, 64)
+    k = torch.zeros(1, 2, 64, 64, dtype=torch.bfloat16)
+    pos = {"t_pos": torch.zeros(1, 64, dtype=torch.long)}
+    with pytest.raises(RuntimeError, match="ROCm GPU only"):
+        cache.upsert_kv(k, k, pos, False)
+    with pytest.raises(RuntimeError, match="ROCm GPU only"):
+        ops.attn_ring(k, cache.kv, cache.written, pos["t_pos"], 128, 1)
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_capi, "_lib", None)
+    monkeypatch.setattr(_capi, "LIB_PATH", "/nonexistent/libwe_attn.so")
+    with pytest.raises(RuntimeError, match="has not been built"):
+        _capi.lib()
+
+
+def test_cache_classes_mirror_reference_interface():
+    cfg = SimpleNamespace(tokens_per_frame=64, local_window=4, global_window=8, global_attn_period=2,
+                          global_attn_offset=1, global_pinned_dilation=2, n_layers=4, n_heads=8,
+                          n_kv_heads=4, d_model=512)
+    c = wea.StaticKVCache(cfg, 1, torch.bfloat16)
+    assert isinstance(c.layers, torch.nn.ModuleList) and len(c.layers) == 4
+    assert [(l.L, l.pinned_dilation, l.num_buckets) for l in c.layers] == [(256, 1, 4), (512, 2, 4), (256, 1, 4), (512, 2, 4)]
+    l0 = c.layers[0]
+    assert l0.kv.shape == (2, 1, 4, 320, 64) and l0.kv.dtype == torch.bfloat16 and l0.capacity == 320 and l0.tpf == 64
+    assert l0.written.dtype == torch.bool and l0.written[256:].all() and not l0.written[:256].any()
+    assert l0.frame_offsets.tolist() == list(range(64)) and l0.current_idx[0] == 256
+    assert len(c.state_dict()) == 0                      # non-persistent buffers, like the reference
+    assert c._is_frozen
+    c.set_frozen(False)
+    assert not c._is_frozen
+    l0.written[:64] = True
+    l0.kv.fill_(1)
+    c.reset()
+    assert c._is_frozen and not l0.kv.any() and not l0.written[:256].any() and l0.written[256:].all()
+    with pytest.raises(AssertionError):
+        wea.LayerKVCache(1, 1, 100, 64, torch.bfloat16, 64)
+    with pytest.raises(AssertionError):
+        wea.LayerKVCache(1, 1, 192, 64, torch.bfloat16, 64, pinned_dilation=2)
+
+
+def test_attention_module_parameters_and_casting():
+    cfg = SimpleNamespace(n_heads=8, n_kv_heads=2, d_model=512, value_residual=True, gated_attn=True)
+    rope = wea.RoPE.one_dimensional(128, 64, 8, 8)
+    split = wea.RingAttn(cfg, 3, rope)
+    assert {"q_proj.weight", "k_proj.weight", "v_proj.weight", "out_proj.weight", "v_lamb", "gate_proj.weight"} == set(split.state_dict())
+    assert split.layer_idx == 3 and split.enable_gqa and split.d_head == 64
+    assert not split.gate_proj.weight.any()
+    merged = wea.RingAttn.from_reference(split, cfg, rope, merged_qkv=True)
+    assert merged.qkv_proj.weight.shape == (512 + 2 * 128, 512)
+    assert torch.equal(merged.qkv_proj.weight[:512], split.q_proj.weight)
+    assert torch.equal(merged.qkv_proj.weight[512:640], split.k_proj.weight)
+    assert torch.equal(merged.out_proj.weight, split.out_proj.weight)
+    merged = merged.to(torch.bfloat16)
+    assert merged.rope.cos.dtype == torch.float32 and merged.qkv_proj.weight.dtype == torch.bfloat16
+    assert rope.cos.shape == (128, 32)
+
+    class Holder(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.config = cfg
+            self.blocks = torch.nn.ModuleList([wea.RingAttn(cfg, i, rope) for i in range(2)])
+
+    class Legacy(wea.RingAttn):
+        pass
+
+    m = Holder()
+    assert wea.install_ring_attention(m, rope, (Legacy,)) == 0
+
+
+def test_custom_ops_registered_with_fake_kernels():
+    q = torch.empty(1, 4, 64, 64, dtype=torch.bfloat16, device="meta")
+    kv = torch.empty(2, 1, 4, 192, 64, dtype=torch.bfloat16, device="meta")
+    written = torch.empty(192, dtype=torch.bool, device="meta")
+    t = torch.empty(1, 64, dtype=torch.long, device="meta")
+    out = torch.ops.world_engine_amd.attn_ring(q, kv, written, t, 128, 1, 0.125)
+    assert out.shape == (1, 4, 64, 64) and out.transpose(1, 2).is_contiguous()
+    tab = torch.empty(64, 32, device="meta")
+    qr = torch.ops.world_engine_amd.rope_kv_store(q, q, q, t, t, t, tab, tab, 8, 8, kv, written, 128, 1, False)
+    assert qr.shape == q.shape

@@ -1,0 +1,337 @@
+"""GPU parity: the HIP path (through the C ABI) against the CPU oracle on identical seeded inputs.
+
+Bars: ring-buffer contents, ``written`` and RoPE outputs bit-exact; attention output within
+max-abs 2e-2 / mean-abs 2e-3 of the fp32 oracle on bf16 inputs.
+"""
+import math
+
+import pytest
+import torch
+
+from oracle import ring_oracle as ro
+from _harness import Pair, assert_attn_close, assert_bits_equal, merged_views, to_dev, MAX_ABS, MEAN_ABS
+import world_engine_amd as wea
+from world_engine_amd import ops
+
+pytestmark = pytest.mark.gpu
+
+
+def _say(msg):
+    print(msg, flush=True)
+
+
+# ------------------------------------------------------------------------------------------
+# RoPE + ring store: bit-exact
+# ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("d", [1, 2, 4])
+@pytest.mark.parametrize("hkv", [4, 2])
+def test_store_bit_exact_over_wraps(gpu_device, dtype, d, hkv):
+    _say(f"store dtype={dtype} d={d} hkv={hkv}")
+    n = 4 * d if d > 1 else 4
+    p = Pair(gpu_device, dtype, B=2, H=4, Hkv=hkv, T=64, Dh=64, n_slots=n, d=d, cfg_id=11)
+    for t in range(3 * n + 2):
+        for sub, frozen in ((0, True), (1, True), (2, False)):
+            p.set_frozen(frozen)
+            q, k, v, pos = p.inputs(t, sub)
+            (q_o, _, _, mask), (q_h, ring) = p.store(q, k, v, pos, strided=(t % 2 == 0))
+            assert_bits_equal(q_h, q_o, f"RoPE(q) t={t} sub={sub}")
+            p.assert_state_equal(what=f"t={t} sub={sub} frozen={frozen}")
+            assert torch.equal(ring.dense().cpu(), mask), f"mask t={t} sub={sub}"
+
+
+def test_store_cfg1_shape_bit_exact(gpu_device):
+    p = Pair(gpu_device, torch.bfloat16, B=1, H=16, Hkv=16, T=256, Dh=128, n_slots=16, cfg_id=1)
+    p.set_frozen(False)
+    for t in (0, 1, 15, 16, 17, 40):
+        q, k, v, pos = p.inputs(t)
+        (q_o, *_), (q_h, _) = p.store(q, k, v, pos)
+        assert_bits_equal(q_h, q_o, f"RoPE(q) t={t}")
+        p.assert_state_equal(what=f"t={t}")
+
+
+def test_reference_signature_upsert_without_rope(gpu_device):
+    """StaticKVCache.upsert(k, v, pos_ids, layer) / LayerKVCache.upsert(kv, pos_ids, frozen) with
+    an already rotated k, as the reference's own attention module would call them."""
+    p = Pair(gpu_device, torch.bfloat16, B=1, H=2, Hkv=2, T=64, Dh=128, n_slots=3, n_layers=2, cfg_id=12)
+    p.set_frozen(False)
+    for t in range(8):
+        q, k, v, pos = p.inputs(t)
+        p.oracle.upsert(k, v, pos, 1)
+        k_all, v_all, ring = p.hip.upsert(k.to(gpu_device), v.to(gpu_device), to_dev(pos, gpu_device), 1)
+        assert k_all.shape == (1, 2, 4 * 64, 128) and k_all.data_ptr() == p.hip.layers[1].kv[0].data_ptr()
+        p.assert_state_equal(layer=1, what=f"t={t}")
+        # layer API with the stacked tensor
+        p.oracle.layers[0].upsert(torch.stack([k, v]), pos, t % 2 == 0)
+        p.hip.layers[0].upsert(torch.stack([k, v]).to(gpu_device), to_dev(pos, gpu_device), t % 2 == 0)
+        p.assert_state_equal(layer=0, what=f"layer api t={t}")
+    p.hip.reset()
+    p.oracle.reset()
+    p.assert_state_equal(layer=0, what="after reset")
+    assert p.hip._is_frozen
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_standalone_rope_bit_exact(gpu_device, dtype):
+    p = Pair(gpu_device, dtype, B=2, H=3, Hkv=3, T=64, Dh=128, n_slots=2, cfg_id=13)
+    q, k, v, pos = p.inputs(5)
+    cos, sin = ro.rope_angles(pos, p.cos, p.sin, p.Hgrid, p.W)
+    got = p.rope(merged_views(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device))[0], to_dev(pos, gpu_device))
+    assert_bits_equal(got, ro.rope_apply(q, cos, sin), "stand-alone RoPE")
+
+
+def test_rope_special_values_round_like_torch(gpu_device):
+    """NaN, infinities, denormals and ties go through the same fp32 -> bf16 rounding as torch."""
+    p = Pair(gpu_device, torch.bfloat16, B=1, H=1, Hkv=1, T=64, Dh=64, n_slots=2, cfg_id=14)
+    q, k, v, pos = p.inputs(1)
+    k[0, 0, 0, :8] = torch.tensor([float("nan"), float("inf"), -float("inf"), 0.0, -0.0, 1e-40, 3.3895e38, -1e-38])
+    (q_o, *_), (q_h, _) = p.store(q, k, v, pos)
+    p.assert_state_equal(what="special values")
+
+
+# ------------------------------------------------------------------------------------------
+# attention
+# ------------------------------------------------------------------------------------------
+def _run_and_check(p, steps, frozen_subs=0, check_steps=None, outlier=False, layer=0, **attn_kw):
+    worst = (0.0, 0.0)
+    for t in range(steps):
+        for sub in range(frozen_subs + 1):
+            frozen = sub < frozen_subs
+            p.set_frozen(frozen)
+            q, k, v, pos = p.inputs(t, sub, outlier)
+            (q_o, k_all, v_all, mask), (q_h, ring) = p.store(q, k, v, pos, layer=layer)
+            out = p.attend(q_h, ring, **attn_kw)
+            p.assert_state_equal(layer=layer, what=f"t={t} sub={sub}")
+            if check_steps is None or t in check_steps:
+                ref = ro.attention_fp32(q_o, k_all, v_all, mask)
+                mx, mean = assert_attn_close(out, ref, f"t={t} sub={sub} kw={attn_kw}")
+                worst = (max(worst[0], mx), max(worst[1], mean))
+    return worst
+
+
+def test_attention_cfg0_shapes_bf16(gpu_device):
+    """BASELINE config 0 geometry (B=1,H=8,Dh=64,T=64, 4 slots, 8 steps) in bf16 on the GPU."""
+    p = Pair(gpu_device, torch.bfloat16, B=1, H=8, Hkv=8, T=64, Dh=64, n_slots=4, cfg_id=0)
+    worst = _run_and_check(p, 8)
+    _say(f"cfg0 shapes: worst max-abs {worst[0]:.2e} mean-abs {worst[1]:.2e}")
+
+
+def test_attention_cfg1_all_32_steps(gpu_device):
+    """BASELINE config 1: B=1,H=16,Dh=128,T=256, 16 slots, 32 steps (warm-up + steady wrap)."""
+    p = Pair(gpu_device, torch.bfloat16, B=1, H=16, Hkv=16, T=256, Dh=128, n_slots=16, cfg_id=1)
+    worst = _run_and_check(p, 32)
+    _say(f"cfg1: worst max-abs {worst[0]:.2e} mean-abs {worst[1]:.2e}")
+
+
+@pytest.mark.parametrize("n_splits", [1, 2, 3, 7, 16])
+@pytest.mark.parametrize("q_tile", [128, 256])
+def test_attention_split_and_tile_variants(gpu_device, n_splits, q_tile):
+    _say(f"variants n_splits={n_splits} q_tile={q_tile}")
+    p = Pair(gpu_device, torch.bfloat16, B=2, H=4, Hkv=2, T=128, Dh=128, n_slots=6, cfg_id=21)
+    _run_and_check(p, 9, n_splits=n_splits, q_tile=q_tile)
+
+
+@pytest.mark.parametrize("dtype,Dh,T", [(torch.float16, 128, 64), (torch.float16, 64, 128),
+                                        (torch.bfloat16, 64, 192), (torch.bfloat16, 128, 320)])
+def test_attention_dtypes_head_dims_and_ragged_tiles(gpu_device, dtype, Dh, T):
+    """T values that are not a multiple of the query tile exercise the partial last tile."""
+    _say(f"dtype={dtype} Dh={Dh} T={T}")
+    p = Pair(gpu_device, dtype, B=1, H=6, Hkv=3, T=T, Dh=Dh, n_slots=3, cfg_id=22)
+    for kw in ({}, {"n_splits": 2, "q_tile": 128}, {"n_splits": 1, "q_tile": 256}):
+        p.hip.reset()
+        p.oracle.reset()
+        _run_and_check(p, 5, **kw)
+
+
+@pytest.mark.parametrize("d", [2, 4])
+def test_attention_with_pinned_dilation(gpu_device, d):
+    p = Pair(gpu_device, torch.bfloat16, B=1, H=2, Hkv=2, T=64, Dh=128, n_slots=4 * d, d=d, cfg_id=23)
+    _run_and_check(p, 4 * d * 2 + 3, frozen_subs=1)
+
+
+def test_attention_cfg2_outlier_channel_three_layers(gpu_device):
+    """BASELINE config 2 semantics (each layer its own ring, K with one x8 channel) on 3 layers."""
+    p = Pair(gpu_device, torch.bfloat16, B=1, H=16, Hkv=16, T=256, Dh=128, n_slots=16, n_layers=3, cfg_id=2)
+    p.set_frozen(False)
+    for t in (0, 1, 2, 17):
+        for layer in range(3):
+            q, k, v, pos = ro.synth_qkv(2, t, layer, 1, 16, 16, 256, 128, torch.bfloat16, outlier=True) + (ro.synth_pos_ids(t, 1, 256, 16),)
+            (q_o, k_all, v_all, mask), (q_h, ring) = p.store(q, k, v, pos, layer=layer)
+            out = p.attend(q_h, ring)
+            p.assert_state_equal(layer=layer, what=f"t={t} layer={layer}")
+            assert_attn_close(out, ro.attention_fp32(q_o, k_all, v_all, mask), f"cfg2 t={t} layer={layer}")
+
+
+def test_attention_cfg4_frozen_substeps_schedule(gpu_device):
+    """BASELINE config 4: 32 slots, 4 frozen substeps re-attending the same ring + 1 persisting
+    call per frame.  State is compared after every call; outputs on the first frames and around
+    the wrap."""
+    p = Pair(gpu_device, torch.bfloat16, B=1, H=16, Hkv=16, T=256, Dh=128, n_slots=32, cfg_id=4)
+    _run_and_check(p, 35, frozen_subs=4, check_steps={0, 1, 31, 32, 34})
+
+
+def test_attention_cfg3_full_size(gpu_device):
+    """BASELINE config 3 at full size (B=4,H=24,T=1024, 8 slots): oracle on three steps, plus
+    size-independent properties on the steady state."""
+    p = Pair(gpu_device, torch.bfloat16, B=4, H=24, Hkv=24, T=1024, Dh=128, n_slots=8, cfg_id=3)
+    _run_and_check(p, 10, check_steps={0, 9})
+    # steady state: permuting the visible slots' contents must not change the result
+    q, k, v, pos = p.inputs(10)
+    p.set_frozen(True)
+    (_, _, _, mask), (q_h, ring) = p.store(q, k, v, pos)
+    base = p.attend(q_h, ring).clone()
+    kv = p.hip.layers[0].kv
+    T = 1024
+    vis = [s for s in range(8) if mask[s * T]]
+    assert len(vis) == 7
+    rolled = kv.clone()
+    for a, b in zip(vis, vis[1:] + vis[:1]):
+        rolled[:, :, :, a * T:(a + 1) * T] = kv[:, :, :, b * T:(b + 1) * T]
+    out2 = ops.attn_ring(q_h, rolled, ring.written, ring.t_pos, ring.L, ring.dilation)
+    d = (out2.float() - base.float()).abs()
+    assert d.max().item() <= 1e-2 and d.mean().item() <= 1e-3
+    # the hidden slot's contents are irrelevant (large finite garbage)
+    hid = [s for s in range(8) if not mask[s * T]][0]
+    rolled.copy_(kv)
+    rolled[:, :, :, hid * T:(hid + 1) * T] = 3e4
+    out3 = ops.attn_ring(q_h, rolled, ring.written, ring.t_pos, ring.L, ring.dilation)
+    assert torch.equal(out3, base)
+    # split count does not matter beyond rounding
+    out4 = p.attend(q_h, ring, n_splits=3)
+    d = (out4.float() - base.float()).abs()
+    assert d.max().item() <= 1e-2 and d.mean().item() <= 1e-3
+
+
+def test_output_layout_and_out_argument(gpu_device):
+    p = Pair(gpu_device, torch.bfloat16, B=2, H=2, Hkv=2, T=64, Dh=64, n_slots=2, cfg_id=24)
+    p.set_frozen(False)
+    q, k, v, pos = p.inputs(0)
+    (q_o, k_all, v_all, mask), (q_h, ring) = p.store(q, k, v, pos)
+    a = p.attend(q_h, ring)
+    assert a.shape == (2, 2, 64, 64) and a.transpose(1, 2).is_contiguous()
+    b = p.attend(q_h, ring, token_major_out=False)
+    assert b.is_contiguous() and torch.equal(a, b)
+    out = torch.empty_like(b)
+    c = p.attend(q_h, ring, out=out)
+    assert c.data_ptr() == out.data_ptr() and torch.equal(out, b)
+
+
+# ------------------------------------------------------------------------------------------
+# module-level drop-in and graph capture
+# ------------------------------------------------------------------------------------------
+def test_ring_attn_module_matches_cpu_composition(gpu_device):
+    """RingAttn.forward (merged QKV, GQA, value residual, head gate) against the same sequence
+    composed on the CPU from torch linears, F.rms_norm and the oracle."""
+    import torch.nn.functional as F
+    from types import SimpleNamespace
+    torch.manual_seed(5)
+    T, H, Hkv, Dh, n = 64, 4, 2, 64, 3
+    cfg = SimpleNamespace(tokens_per_frame=T, local_window=n, global_window=n, global_attn_period=1,
+                          global_pinned_dilation=1, n_layers=1, n_heads=H, n_kv_heads=Hkv, d_model=H * Dh,
+                          value_residual=True, gated_attn=True)
+    cos, sin = ro.rope_table_1d(16 * T, Dh)
+    rope = wea.RoPE(cos, sin, 8, 8)
+    mod = wea.RingAttn(cfg, 0, rope, merged_qkv=True)
+    with torch.no_grad():
+        mod.gate_proj.weight.normal_(0, 0.5)
+    mod = mod.to(torch.bfloat16)
+    cpu_sd = {k: v.clone() for k, v in mod.state_dict().items()}
+    mod = mod.to(gpu_device)
+    cache = wea.StaticKVCache(cfg, 1, torch.bfloat16).to(gpu_device)
+    ocache = ro.OracleStaticKVCache(cfg, 1, torch.bfloat16)
+    v1_h = v1_o = None
+    for t in range(5):
+        frozen = t % 2 == 1
+        cache.set_frozen(frozen)
+        ocache.set_frozen(frozen)
+        x = torch.randn(1, T, H * Dh).to(torch.bfloat16)
+        pos = ro.synth_pos_ids(t, 1, T, 8)
+        y_h, v1_h = mod(x.to(gpu_device), to_dev(pos, gpu_device), v1_h, cache)
+        # CPU composition
+        qkv = F.linear(x, cpu_sd["qkv_proj.weight"])
+        q, k, v = qkv.split((H * Dh, Hkv * Dh, Hkv * Dh), dim=-1)
+        q = q.reshape(1, T, H, Dh).transpose(1, 2)
+        k = k.reshape(1, T, Hkv, Dh).transpose(1, 2)
+        v = v.reshape(1, T, Hkv, Dh).transpose(1, 2)
+        v1_o = v if v1_o is None else v1_o
+        v = torch.lerp(v, v1_o.view_as(v), cpu_sd["v_lamb"])
+        q, k = F.rms_norm(q, (Dh,)), F.rms_norm(k, (Dh,))
+        y, _ = ro.layer_step(ocache, 0, q, k, v, pos, cos, sin, 8, 8)
+        gates = torch.sigmoid(F.linear(x[..., :H], cpu_sd["gate_proj.weight"]))
+        y = y * gates.permute(0, 2, 1).unsqueeze(-1)
+        y_o = F.linear(y.transpose(1, 2).reshape(1, T, -1), cpu_sd["out_proj.weight"])
+        d = (y_h.float().cpu() - y_o.float()).abs()
+        assert d.max().item() < 3e-2 and d.mean().item() < 3e-3, (t, d.max().item(), d.mean().item())
+        assert torch.equal(cache.layers[0].written.cpu(), ocache.layers[0].written)
+
+
+def test_hip_graph_replay_matches_eager(gpu_device):
+    """One frame step (store + attention) captured in a HIP graph and replayed for successive
+    frames by updating only device tensors; every replay must equal the eager result."""
+    p = Pair(gpu_device, torch.bfloat16, B=1, H=4, Hkv=4, T=128, Dh=128, n_slots=4, cfg_id=25)
+    p.set_frozen(False)
+    eager = Pair(gpu_device, torch.bfloat16, B=1, H=4, Hkv=4, T=128, Dh=128, n_slots=4, cfg_id=25)
+    eager.set_frozen(False)
+    dev = gpu_device
+    qs, ks, vs = (torch.empty(1, 4, 128, 128, dtype=torch.bfloat16, device=dev) for _ in range(3))
+    pos_s = to_dev(ro.synth_pos_ids(0, 1, 128, p.W), dev)
+    layer = p.hip.layers[0]
+    out_s = torch.empty(1, 4, 128, 128, dtype=torch.bfloat16, device=dev)
+    n_splits = 2
+    ws = torch.empty(ops.attn_workspace_bytes(1, 4, 128, 128, n_splits), dtype=torch.uint8, device=dev)
+
+    def step():
+        q_rot = ops.rope_kv_store(qs, ks, vs, pos_s, p.rope.cos, p.rope.sin, p.Hgrid, p.W, layer.kv,
+                                  layer.written, layer.L, 1, False)
+        ops.attn_ring(q_rot, layer.kv, layer.written, pos_s["t_pos"], layer.L, 1, n_splits=n_splits,
+                      out=out_s, workspace=ws)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                               # warm-up outside capture
+    torch.cuda.current_stream().wait_stream(side)
+    layer.reset()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    layer.reset()
+    for t in range(10):
+        q, k, v, pos = p.inputs(t)
+        qs.copy_(q); ks.copy_(k); vs.copy_(v)
+        pos_s["t_pos"].fill_(t)
+        graph.replay()
+        torch.cuda.synchronize()
+        (_, _, _, _), (q_h, ring) = eager.store(q, k, v, pos, strided=False)
+        ref = eager.attend(q_h, ring, n_splits=n_splits, token_major_out=False)
+        assert torch.equal(out_s, ref), f"replay {t} differs from eager"
+        assert torch.equal(layer.kv, eager.hip.layers[0].kv) and torch.equal(layer.written, eager.hip.layers[0].written)
+
+
+# ------------------------------------------------------------------------------------------
+# error behaviour through the C ABI
+# ------------------------------------------------------------------------------------------
+def test_bad_inputs_raise(gpu_device):
+    p = Pair(gpu_device, torch.bfloat16, B=1, H=2, Hkv=2, T=64, Dh=64, n_slots=2, cfg_id=26)
+    q, k, v, pos = p.inputs(0)
+    dev = gpu_device
+    with pytest.raises(RuntimeError, match="one frame per upsert"):
+        p.hip.upsert(k[:, :, :32].to(dev), v[:, :, :32].to(dev), to_dev(pos, dev), 0)
+    p.hip.layers[0].check_inputs = True
+    bad = to_dev(pos, dev)
+    bad["t_pos"] = bad["t_pos"].clone()
+    bad["t_pos"][0, 3] = 7
+    with pytest.raises(RuntimeError, match="constant within frame"):
+        p.hip.upsert(k.to(dev), v.to(dev), bad, 0)
+    bad["t_pos"].fill_(-1)
+    with pytest.raises(RuntimeError, match="non-negative"):
+        p.hip.upsert(k.to(dev), v.to(dev), bad, 0)
+    # unsupported head dim for the attention kernel
+    layer = wea.LayerKVCache(1, 1, 64, 32, torch.bfloat16, 64).to(dev)
+    with pytest.raises(RuntimeError, match="not covered"):
+        ops.attn_ring(torch.zeros(1, 1, 64, 32, dtype=torch.bfloat16, device=dev), layer.kv, layer.written,
+                      torch.zeros(1, 64, dtype=torch.long, device=dev), 64, 1)
+    with pytest.raises(RuntimeError, match="not covered"):
+        lay32 = wea.LayerKVCache(1, 1, 128, 64, torch.float32, 64).to(dev)
+        ops.attn_ring(torch.zeros(1, 1, 64, 64, dtype=torch.float32, device=dev), lay32.kv, lay32.written,
+                      torch.zeros(1, 64, dtype=torch.long, device=dev), 128, 1)

@@ -1,0 +1,82 @@
+"""ctypes binding of the C ABI declared in ``include/we_attn.h``.
+
+The shared library is built in-tree by ``world_engine_amd/build.py`` (``hipcc`` for gfx950).
+There is no fallback: if the library is missing, every call raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_float, c_int32, c_int64, c_size_t, c_void_p, POINTER
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libwe_attn.so")
+
+WE_DTYPE_BF16, WE_DTYPE_F16, WE_DTYPE_F32 = 0, 1, 2
+WE_MAX_SLOTS = 256
+
+_I64x3 = POINTER(c_int64)
+
+# name -> (restype, argtypes); must list every symbol include/we_attn.h declares
+SIGNATURES = {
+    "we_version": (c_int32, []),
+    "we_error_string": (c_char_p, [c_int32]),
+    "we_rope_kv_store": (c_int32, [
+        c_void_p, c_void_p, c_void_p,              # q, k, v
+        _I64x3, _I64x3, _I64x3,                    # strides
+        c_void_p,                                  # q_out
+        c_void_p, c_void_p, c_int64,               # cos, sin, table_rows
+        c_void_p, c_void_p, c_void_p,              # t_pos, y_pos, x_pos
+        c_int64, c_int64, c_int64,                 # pos_stride_b, grid_h, grid_w
+        c_void_p, c_void_p,                        # kv, written
+        c_int32, c_int32, c_int32, c_int32, c_int32, c_int64,   # B H Hkv T Dh L
+        c_int32, c_int32, c_int32, c_void_p,       # dilation, is_frozen, dtype, stream
+    ]),
+    "we_rope_apply": (c_int32, [
+        c_void_p, _I64x3, c_void_p,                # x, strides, x_out
+        c_void_p, c_void_p, c_int64,               # cos, sin, table_rows
+        c_void_p, c_void_p, c_void_p,              # t_pos, y_pos, x_pos
+        c_int64, c_int64, c_int64,                 # pos_stride_b, grid_h, grid_w
+        c_int32, c_int32, c_int32, c_int32,        # B H T Dh
+        c_int32, c_void_p,                         # dtype, stream
+    ]),
+    "we_attn_auto_splits": (c_int32, [c_int32, c_int32, c_int32, c_int32, c_int32, c_int64]),
+    "we_attn_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32, c_int32]),
+    "we_attn_ring_fwd": (c_int32, [
+        c_void_p, _I64x3,                          # q, q_strides
+        c_void_p, c_void_p, c_void_p,              # kv, written, t_pos
+        c_void_p, _I64x3,                          # out, out_strides
+        c_void_p, c_size_t,                        # workspace, bytes
+        c_int32, c_int32, c_int32, c_int32, c_int32, c_int64,   # B H Hkv T Dh L
+        c_int32, c_float, c_int32, c_int32, c_int32, c_void_p,  # dilation scale n_splits q_tile dtype stream
+    ]),
+}
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    """Load the library once; raise if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: the HIP extension has not been built "
+                "(run `python -m world_engine_amd.build`). There is no CPU or PyTorch fallback."
+            )
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = handle
+    return _lib
+
+
+def check(code: int, what: str) -> None:
+    if code != 0:
+        msg = lib().we_error_string(code).decode()
+        raise RuntimeError(f"{what} failed: {msg} (code {code})")
+
+
+def i64x3(a: int, b: int, c: int):
+    return (c_int64 * 3)(a, b, c)

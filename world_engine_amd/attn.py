@@ -1,0 +1,165 @@
+"""Self-attention module with the reference's ``forward(x, pos_ids, v1, kv_cache)`` contract.
+
+``RingAttn`` takes the place of ``Attn`` / ``MergedQKVAttn`` (``src/model/attn.py:70-122``,
+``src/patch_model.py:92-141``): same parameters and state-dict keys, same call signature, same
+order of operations.  The part between the q/k/v projection and the output projection - RoPE,
+cache update, masked attention - runs as two HIP kernel launches (three with context splits)
+instead of the reference's eager/compiled op sequence.  Projections, the weightless RMS norm,
+the value-residual lerp and the head gate stay ordinary torch ops; they are the neighbours of
+the path, not the path.
+"""
+from __future__ import annotations
+
+import math
+from typing import Mapping, Optional
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor, nn
+
+from . import ops
+from .kv_cache import RingMask
+
+
+class RoPE(nn.Module):
+    """Table-driven rotary embedding (``src/model/attn.py:12-40``).  ``cos``/``sin`` are fp32
+    ``[n_frames*height*width, Dh/2]`` buffers that ignore dtype casts of the parent model (the
+    reference keeps them fp32 through ``NoCastModule``); the row of token ``(t, y, x)`` is
+    ``t*height*width + y*width + x``."""
+
+    def __init__(self, cos: Tensor, sin: Tensor, height: int, width: int):
+        super().__init__()
+        if cos.dtype != torch.float32 or sin.dtype != torch.float32 or cos.shape != sin.shape:
+            raise AssertionError("RoPE tables must be fp32 and of equal shape")
+        self.height, self.width = height, width
+        self.register_buffer("cos", cos.contiguous(), persistent=False)
+        self.register_buffer("sin", sin.contiguous(), persistent=False)
+
+    def _apply(self, fn, *args, **kwargs):
+        def keep_dtype(t):
+            out = fn(t)
+            return out if out.dtype == t.dtype else out.to(dtype=t.dtype)
+        return super()._apply(keep_dtype, *args, **kwargs)
+
+    @classmethod
+    def one_dimensional(cls, n_rows: int, d_head: int, height: int, width: int, base: float = 10000.0):
+        """1-D rotary table over the absolute token position: ``angle[p,i] = p * base**(-2i/Dh)``
+        (computed in fp64, stored fp32)."""
+        inv = torch.pow(torch.tensor(base, dtype=torch.float64),
+                        -2.0 * torch.arange(d_head // 2, dtype=torch.float64) / d_head)
+        ang = torch.arange(n_rows, dtype=torch.float64)[:, None] * inv[None, :]
+        return cls(ang.cos().float(), ang.sin().float(), height, width)
+
+    def forward(self, x: Tensor, pos_ids: Mapping[str, Tensor]) -> Tensor:
+        return ops.rope_apply(x, pos_ids, self.cos, self.sin, self.height, self.width)
+
+
+def ring_attention(q: Tensor, k: Tensor, v: Tensor, block_mask: RingMask, enable_gqa: bool = False,
+                   scale: Optional[float] = None) -> Tensor:
+    """Call-compatible stand-in for ``flex_attention(q, k, v, block_mask=bm, enable_gqa=...)`` at
+    ``src/model/attn.py:116``: ``k``/``v`` must be the cache planes that ``upsert`` returned
+    together with ``block_mask``."""
+    kv = block_mask.kv
+    if k.data_ptr() != kv[0].data_ptr() or v.data_ptr() != kv[1].data_ptr():
+        raise RuntimeError("ring_attention needs the k/v views returned by the cache's upsert")
+    if not enable_gqa and q.shape[1] != k.shape[1]:
+        raise RuntimeError("query and key head counts differ but enable_gqa is False")
+    return ops.attn_ring(q, kv, block_mask.written, block_mask.t_pos, block_mask.L,
+                         block_mask.dilation, scale)
+
+
+class RingAttn(nn.Module):
+    """Drop-in for the reference's attention module.
+
+    ``config`` provides ``d_model, n_heads`` and optionally ``n_kv_heads, value_residual,
+    gated_attn`` (``src/model/attn.py:76-96``).  ``rope`` is a shared :class:`RoPE`.  With
+    ``merged_qkv`` the three projections are one ``qkv_proj`` as after the reference's inference
+    patch (``src/patch_model.py:102-114``); otherwise the keys are ``q_proj/k_proj/v_proj``.
+    """
+
+    def __init__(self, config, layer_idx: int, rope: RoPE, merged_qkv: bool = False):
+        super().__init__()
+        self.config = config
+        self.layer_idx = layer_idx
+        self.n_heads = config.n_heads
+        self.n_kv_heads = getattr(config, "n_kv_heads", config.n_heads)
+        if config.d_model % self.n_heads != 0:
+            raise AssertionError("d_model must be divisible by n_heads")
+        self.d_head = config.d_model // self.n_heads
+        self.enable_gqa = self.n_heads != self.n_kv_heads
+        self.q_out = self.n_heads * self.d_head
+        self.kv_out = self.n_kv_heads * self.d_head
+
+        self.value_residual = getattr(config, "value_residual", False)
+        if self.value_residual:
+            self.v_lamb = nn.Parameter(torch.tensor(0.5))
+
+        self.merged_qkv = merged_qkv
+        if merged_qkv:
+            self.qkv_proj = nn.Linear(config.d_model, self.q_out + 2 * self.kv_out, bias=False)
+        else:
+            self.q_proj = nn.Linear(config.d_model, self.q_out, bias=False)
+            self.k_proj = nn.Linear(config.d_model, self.kv_out, bias=False)
+            self.v_proj = nn.Linear(config.d_model, self.kv_out, bias=False)
+        self.out_proj = nn.Linear(config.d_model, config.d_model, bias=False)
+        self.rope = rope
+
+        self.gated_attn = getattr(config, "gated_attn", False)
+        if self.gated_attn:
+            self.gate_proj = nn.Linear(self.n_heads, self.n_heads, bias=False)
+            nn.init.zeros_(self.gate_proj.weight)
+
+    @classmethod
+    def from_reference(cls, src: nn.Module, config, rope: RoPE, merged_qkv: bool = True):
+        """Build from an ``Attn``-like module (anything with ``layer_idx`` and a matching state
+        dict), the way the reference's ``MergedQKVAttn(src, config)`` does."""
+        new = cls(config, src.layer_idx, rope, merged_qkv=merged_qkv)
+        ref_w = next(src.parameters())
+        new.to(device=ref_w.device, dtype=ref_w.dtype)
+        state = {k: v for k, v in src.state_dict().items()}
+        if merged_qkv and "q_proj.weight" in state:
+            state["qkv_proj.weight"] = torch.cat(
+                [state.pop("q_proj.weight"), state.pop("k_proj.weight"), state.pop("v_proj.weight")], dim=0)
+        new.load_state_dict(state, strict=False)
+        new.train(src.training)
+        return new
+
+    def forward(self, x: Tensor, pos_ids: Mapping[str, Tensor], v1: Optional[Tensor], kv_cache):
+        B, T = x.shape[:2]
+        if self.merged_qkv:
+            q, k, v = self.qkv_proj(x).split((self.q_out, self.kv_out, self.kv_out), dim=-1)
+        else:
+            q, k, v = self.q_proj(x), self.k_proj(x), self.v_proj(x)
+        q = q.reshape(B, T, self.n_heads, self.d_head).transpose(1, 2)
+        k = k.reshape(B, T, self.n_kv_heads, self.d_head).transpose(1, 2)
+        v = v.reshape(B, T, self.n_kv_heads, self.d_head).transpose(1, 2)
+
+        if self.value_residual:
+            v1 = v if v1 is None else v1
+            v = torch.lerp(v, v1.view_as(v), self.v_lamb)
+
+        q = F.rms_norm(q, (self.d_head,))
+        k = F.rms_norm(k, (self.d_head,))
+
+        # RoPE(q), RoPE(k), cache write: one launch.  Attention over the ring: one or two.
+        q, k_all, v_all, ring = kv_cache.rope_upsert(q, k, v, pos_ids, self.rope, self.layer_idx)
+        y = ring_attention(q, k_all, v_all, ring, enable_gqa=self.enable_gqa)
+
+        if self.gated_attn:
+            gates = torch.sigmoid(self.gate_proj(x[..., : self.n_heads]))
+            y = y * gates.permute(0, 2, 1).unsqueeze(-1)
+
+        y = y.transpose(1, 2).reshape(B, T, -1)
+        return self.out_proj(y), v1
+
+
+def install_ring_attention(model: nn.Module, rope: RoPE, attn_types: tuple, merged_qkv: bool = True) -> int:
+    """Swap every submodule that is an instance of ``attn_types`` for a :class:`RingAttn`, the
+    same ``set_submodule`` walk the reference uses for its merged-QKV patch
+    (``src/patch_model.py:144-147``).  Returns the number of modules replaced."""
+    n = 0
+    for name, mod in list(model.named_modules()):
+        if isinstance(mod, attn_types) and not isinstance(mod, RingAttn):
+            model.set_submodule(name, RingAttn.from_reference(mod, model.config, rope, merged_qkv))
+            n += 1
+    return n

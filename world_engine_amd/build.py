@@ -1,0 +1,37 @@
+"""Build ``libwe_attn.so`` (HIP, gfx950) in-tree: ``python -m world_engine_amd.build``."""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+SOURCES = ["rope_kv_store.hip", "attn_ring.hip", "capi.hip"]
+OUT = os.path.join(HERE, "libwe_attn.so")
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    # keep fp32 arithmetic scalar: packed fp32 instructions are avoided on purpose
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def build(verbose: bool = False) -> str:
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc, *HIPCC_FLAGS, *[os.path.join(CSRC, s) for s in SOURCES], "-o", OUT]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "packed-fp32-ops"
+    err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({res.returncode}):\n{err}")
+    if verbose and err.strip():
+        print(err, file=sys.stderr)
+    return OUT
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

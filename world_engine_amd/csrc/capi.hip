@@ -1,0 +1,200 @@
+// C ABI of the ring-buffer attention library: argument validation and kernel dispatch.
+// Declarations and the reference call sites each entry point replaces: include/we_attn.h.
+#include "../../include/we_attn.h"
+#include "we_kernels.h"
+
+namespace {
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int elem_bytes(int dtype) { return dtype == WE_DTYPE_F32 ? 4 : 2; }
+
+// element strides whose byte value keeps every row start 16-byte aligned
+bool strides_ok(const int64_t s[3], int dtype) {
+  const int per16 = 16 / elem_bytes(dtype);
+  return s[0] % per16 == 0 && s[1] % per16 == 0 && s[2] % per16 == 0;
+}
+
+int ring_shape_ok(int B, int H, int Hkv, int T, int Dh, int64_t L, int dilation) {
+  if (B <= 0 || H <= 0 || Hkv <= 0 || T <= 0 || Dh <= 0 || L <= 0 || dilation <= 0) return WE_ERR_BAD_SHAPE;
+  if (H % Hkv != 0 || L % T != 0 || (L / T) % dilation != 0) return WE_ERR_BAD_SHAPE;
+  return WE_OK;
+}
+
+struct AttnPlan {
+  int variant;   // 1: 128 queries per workgroup, 2: 256
+  int n_splits;
+};
+
+// Pick the query-tile size and the number of context splits so that the grid fills the 256 CUs
+// (two 128-query workgroups or one 256-query workgroup fit per CU) without making a split
+// shorter than two 64-key tiles of the steady-state context.
+AttnPlan plan_attn(int B, int H, int T, int64_t L, int n_splits, int variant) {
+  AttnPlan pl;
+  const int64_t wg256 = (int64_t)B * H * ((T + 255) / 256);
+  pl.variant = variant ? variant : ((wg256 >= 256 && T >= 256) ? 2 : 1);
+  if (n_splits > 0) {
+    pl.n_splits = n_splits;
+    return pl;
+  }
+  const int bm = pl.variant == 2 ? 256 : 128;
+  const int64_t base = (int64_t)B * H * ((T + bm - 1) / bm);
+  const int64_t slots_per_cu = pl.variant == 2 ? 1 : 2;
+  const int64_t want = 256 * slots_per_cu;
+  int s = 1;
+  if (base < want) {
+    s = (int)((want + base - 1) / base);
+    const int64_t tiles = L / 64;  // visible tiles at steady state
+    const int64_t max_s = tiles / 2 > 0 ? tiles / 2 : 1;
+    if (s > max_s) s = (int)max_s;
+    if (s > 64) s = 64;
+  }
+  pl.n_splits = s;
+  return pl;
+}
+
+}  // namespace
+
+extern "C" {
+
+int we_version(void) { return 100; }
+
+const char* we_error_string(int code) {
+  switch (code) {
+    case WE_OK: return "ok";
+    case WE_ERR_NULL_POINTER: return "required pointer is NULL";
+    case WE_ERR_BAD_SHAPE: return "inconsistent sizes (need sizes > 0, H % Hkv == 0, L % T == 0, (L/T) % dilation == 0)";
+    case WE_ERR_UNSUPPORTED: return "head dim, frame length, slot count or dtype not covered by the kernels";
+    case WE_ERR_ALIGNMENT: return "pointer or stride breaks 16-byte alignment";
+    case WE_ERR_WORKSPACE: return "split-context workspace missing or too small";
+    case WE_ERR_LAUNCH: return "HIP runtime refused the kernel launch";
+    default: return "unknown error code";
+  }
+}
+
+int we_rope_kv_store(const void* q, const void* k, const void* v, const int64_t q_strides[3],
+                     const int64_t k_strides[3], const int64_t v_strides[3], void* q_out,
+                     const float* cos_table, const float* sin_table, int64_t table_rows,
+                     const int64_t* t_pos, const int64_t* y_pos, const int64_t* x_pos,
+                     int64_t pos_stride_b, int64_t grid_h, int64_t grid_w, void* kv, uint8_t* written,
+                     int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L,
+                     int32_t dilation, int32_t is_frozen, int32_t dtype, void* stream) {
+  if (!k || !v || !k_strides || !v_strides || !t_pos || !kv || !written) return WE_ERR_NULL_POINTER;
+  if ((q == nullptr) != (q_out == nullptr)) return WE_ERR_NULL_POINTER;
+  if (q && !q_strides) return WE_ERR_NULL_POINTER;
+  if ((cos_table == nullptr) != (sin_table == nullptr)) return WE_ERR_NULL_POINTER;
+  if (cos_table && (!y_pos || !x_pos)) return WE_ERR_NULL_POINTER;
+  if (dtype != WE_DTYPE_BF16 && dtype != WE_DTYPE_F16 && dtype != WE_DTYPE_F32) return WE_ERR_UNSUPPORTED;
+  int rc = ring_shape_ok(B, H, Hkv, T, Dh, L, dilation);
+  if (rc != WE_OK) return rc;
+  if (Dh % 16 != 0) return WE_ERR_UNSUPPORTED;
+  if (cos_table && (table_rows <= 0 || grid_h <= 0 || grid_w <= 0)) return WE_ERR_BAD_SHAPE;
+  if (!aligned16(k) || !aligned16(v) || !aligned16(kv) || (q && (!aligned16(q) || !aligned16(q_out))) ||
+      (cos_table && (!aligned16(cos_table) || !aligned16(sin_table))))
+    return WE_ERR_ALIGNMENT;
+  if (!strides_ok(k_strides, dtype) || !strides_ok(v_strides, dtype) || (q && !strides_ok(q_strides, dtype)))
+    return WE_ERR_ALIGNMENT;
+
+  we::StoreParams p;
+  p.q = q; p.k = k; p.v = v; p.q_out = q_out; p.kv = kv; p.written = written;
+  p.cos_t = cos_table; p.sin_t = sin_table;
+  p.t_pos = t_pos; p.y_pos = y_pos; p.x_pos = x_pos;
+  p.qs_b = q ? q_strides[0] : 0; p.qs_h = q ? q_strides[1] : 0; p.qs_t = q ? q_strides[2] : 0;
+  p.ks_b = k_strides[0]; p.ks_h = k_strides[1]; p.ks_t = k_strides[2];
+  p.vs_b = v_strides[0]; p.vs_h = v_strides[1]; p.vs_t = v_strides[2];
+  p.pos_stride_b = pos_stride_b;
+  p.table_rows = table_rows;
+  p.grid_hw = grid_h * grid_w; p.grid_w = grid_w;
+  p.L = L;
+  p.B = B; p.H = H; p.Hkv = Hkv; p.T = T; p.Dh = Dh;
+  p.dilation = dilation; p.num_buckets = (int)((L / T) / dilation); p.frozen = is_frozen ? 1 : 0;
+  return we::launch_rope_kv_store(p, dtype, static_cast<hipStream_t>(stream)) == hipSuccess ? WE_OK : WE_ERR_LAUNCH;
+}
+
+int we_rope_apply(const void* x, const int64_t x_strides[3], void* x_out, const float* cos_table,
+                  const float* sin_table, int64_t table_rows, const int64_t* t_pos, const int64_t* y_pos,
+                  const int64_t* x_pos, int64_t pos_stride_b, int64_t grid_h, int64_t grid_w, int32_t B,
+                  int32_t H, int32_t T, int32_t Dh, int32_t dtype, void* stream) {
+  if (!x || !x_strides || !x_out || !cos_table || !sin_table || !t_pos || !y_pos || !x_pos)
+    return WE_ERR_NULL_POINTER;
+  if (dtype != WE_DTYPE_BF16 && dtype != WE_DTYPE_F16 && dtype != WE_DTYPE_F32) return WE_ERR_UNSUPPORTED;
+  if (B <= 0 || H <= 0 || T <= 0 || Dh <= 0 || table_rows <= 0 || grid_h <= 0 || grid_w <= 0)
+    return WE_ERR_BAD_SHAPE;
+  if (Dh % 16 != 0) return WE_ERR_UNSUPPORTED;
+  if (!aligned16(x) || !aligned16(x_out) || !aligned16(cos_table) || !aligned16(sin_table) ||
+      !strides_ok(x_strides, dtype))
+    return WE_ERR_ALIGNMENT;
+  we::StoreParams p = {};
+  p.q = x; p.q_out = x_out;
+  p.cos_t = cos_table; p.sin_t = sin_table;
+  p.t_pos = t_pos; p.y_pos = y_pos; p.x_pos = x_pos;
+  p.qs_b = x_strides[0]; p.qs_h = x_strides[1]; p.qs_t = x_strides[2];
+  p.pos_stride_b = pos_stride_b;
+  p.table_rows = table_rows;
+  p.grid_hw = grid_h * grid_w; p.grid_w = grid_w;
+  p.L = T;
+  p.B = B; p.H = H; p.Hkv = 0; p.T = T; p.Dh = Dh;
+  p.dilation = 1; p.num_buckets = 1; p.frozen = 1;
+  return we::launch_rope_kv_store(p, dtype, static_cast<hipStream_t>(stream)) == hipSuccess ? WE_OK : WE_ERR_LAUNCH;
+}
+
+int32_t we_attn_auto_splits(int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L) {
+  (void)Hkv; (void)Dh;
+  if (B <= 0 || H <= 0 || T <= 0 || L <= 0) return 1;
+  return plan_attn(B, H, T, L, 0, 0).n_splits;
+}
+
+size_t we_attn_workspace_bytes(int32_t B, int32_t H, int32_t T, int32_t Dh, int32_t n_splits) {
+  if (n_splits <= 1 || B <= 0 || H <= 0 || T <= 0 || Dh <= 0) return 0;
+  const size_t rows = (size_t)B * H * T;
+  return (size_t)n_splits * rows * ((size_t)Dh + 2) * sizeof(float);
+}
+
+int we_attn_ring_fwd(const void* q, const int64_t q_strides[3], const void* kv, const uint8_t* written,
+                     const int64_t* t_pos, void* out, const int64_t out_strides[3], void* workspace,
+                     size_t workspace_bytes, int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh,
+                     int64_t L, int32_t dilation, float scale, int32_t n_splits, int32_t q_tile,
+                     int32_t dtype, void* stream) {
+  if (!q || !q_strides || !kv || !written || !t_pos || !out || !out_strides) return WE_ERR_NULL_POINTER;
+  int rc = ring_shape_ok(B, H, Hkv, T, Dh, L, dilation);
+  if (rc != WE_OK) return rc;
+  if (dtype != WE_DTYPE_BF16 && dtype != WE_DTYPE_F16) return WE_ERR_UNSUPPORTED;
+  if (Dh != 64 && Dh != 128) return WE_ERR_UNSUPPORTED;
+  if (T % 64 != 0 || L / T > WE_MAX_SLOTS) return WE_ERR_UNSUPPORTED;
+  if (!(scale > 0.f) || n_splits < 0 || n_splits > 64) return WE_ERR_BAD_SHAPE;
+  if (q_tile != 0 && q_tile != 128 && q_tile != 256) return WE_ERR_UNSUPPORTED;
+  if (!aligned16(q) || !aligned16(kv) || !aligned16(out) || !strides_ok(q_strides, dtype) ||
+      !strides_ok(out_strides, dtype))
+    return WE_ERR_ALIGNMENT;
+
+  const int variant = q_tile == 0 ? 0 : (q_tile == 256 ? 2 : 1);
+  const AttnPlan pl = plan_attn(B, H, T, L, n_splits, variant);
+  if (pl.n_splits > 1) {
+    if (!workspace || !aligned16(workspace)) return WE_ERR_WORKSPACE;
+    if (workspace_bytes < we_attn_workspace_bytes(B, H, T, Dh, pl.n_splits)) return WE_ERR_WORKSPACE;
+  }
+
+  we::AttnParams p;
+  p.q = q; p.kv = kv; p.written = written; p.t_pos = t_pos; p.out = out;
+  const size_t rows = (size_t)B * H * T;
+  p.ws_o = static_cast<float*>(workspace);
+  p.ws_ml = p.ws_o ? p.ws_o + (size_t)pl.n_splits * rows * Dh : nullptr;
+  p.qs_b = q_strides[0]; p.qs_h = q_strides[1]; p.qs_t = q_strides[2];
+  p.os_b = out_strides[0]; p.os_h = out_strides[1]; p.os_t = out_strides[2];
+  p.L = L;
+  p.B = B; p.H = H; p.Hkv = Hkv; p.T = T;
+  p.n_slots = (int)(L / T); p.dilation = dilation; p.num_buckets = p.n_slots / dilation;
+  p.n_splits = pl.n_splits;
+  const int bm = we::attn_block_m(Dh, pl.variant);
+  p.q_tiles = (T + bm - 1) / bm;
+  p.members = (H / Hkv) * p.q_tiles;
+  p.unit_splits = B * Hkv * pl.n_splits;
+  p.scale_log2 = scale * 1.4426950408889634f;
+
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (we::launch_attn_ring(p, Dh, dtype, pl.variant, st) != hipSuccess) return WE_ERR_LAUNCH;
+  if (pl.n_splits > 1 && we::launch_attn_combine(p, Dh, dtype, st) != hipSuccess) return WE_ERR_LAUNCH;
+  return WE_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,59 @@
+// Kernel parameter blocks and host-side launchers shared by the C ABI translation unit.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace we {
+
+struct StoreParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* q_out;
+  void* kv;
+  uint8_t* written;
+  const float* cos_t;
+  const float* sin_t;
+  const int64_t* t_pos;
+  const int64_t* y_pos;
+  const int64_t* x_pos;
+  int64_t qs_b, qs_h, qs_t;  // element strides
+  int64_t ks_b, ks_h, ks_t;
+  int64_t vs_b, vs_h, vs_t;
+  int64_t pos_stride_b;
+  int64_t table_rows;
+  int64_t grid_hw, grid_w;
+  int64_t L;
+  int B, H, Hkv, T, Dh;
+  int dilation, num_buckets, frozen;
+};
+
+struct AttnParams {
+  const void* q;
+  const void* kv;
+  const uint8_t* written;
+  const int64_t* t_pos;
+  void* out;
+  float* ws_o;   // [n_splits][B*H*T][Dh] unnormalised partial outputs
+  float* ws_ml;  // [n_splits][B*H*T][2]  running max (log2 domain) and sum
+  int64_t qs_b, qs_h, qs_t;
+  int64_t os_b, os_h, os_t;
+  int64_t L;
+  int B, H, Hkv, T;
+  int n_slots, dilation, num_buckets;
+  int n_splits;
+  int q_tiles;      // ceil(T / queries per workgroup)
+  int members;      // workgroups that share one K/V stream: (H/Hkv) * q_tiles
+  int unit_splits;  // B * Hkv * n_splits
+  float scale_log2; // softmax scale * log2(e)
+};
+
+hipError_t launch_rope_kv_store(const StoreParams& p, int dtype, hipStream_t stream);
+
+// queries handled by one workgroup of the attention kernel for a head dim / variant
+int attn_block_m(int Dh, int variant);
+hipError_t launch_attn_ring(const AttnParams& p, int Dh, int dtype, int variant, hipStream_t stream);
+hipError_t launch_attn_combine(const AttnParams& p, int Dh, int dtype, hipStream_t stream);
+
+}  // namespace we

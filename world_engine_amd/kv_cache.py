@@ -1,0 +1,148 @@
+"""Ring-buffer KV cache with the reference's class interface, backed by the HIP kernels.
+
+Interface kept from ``src/model/kv_cache.py`` of world_engine: ``LayerKVCache(B, H, L, Dh, dtype,
+tokens_per_frame, pinned_dilation)`` with buffers ``kv`` ``[2,B,H,L+T,Dh]``, ``written``
+``[L+T]``, ``frame_offsets``, ``current_idx`` and methods ``reset`` / ``upsert`` (:64-154);
+``StaticKVCache(config, batch_size, dtype)`` with ``layers``, ``reset``, ``set_frozen``,
+``upsert(k, v, pos_ids, layer)`` (:157-193).  After every call ``kv`` and ``written`` hold
+exactly the bits the reference's buffers would.
+
+What differs by design: ``upsert`` returns a :class:`RingMask` (a view of the cache state) where
+the reference returns a flex-attention ``BlockMask`` (:12-61, :144).  The only consumer of that
+object in the reference is the attention call this package also replaces.  The cache writes are
+one fused kernel launch; the slot is computed on the device from ``t_pos[0, 0]`` (:126-131), so
+no host synchronisation happens outside the optional eager input checks (:112-124).
+"""
+from __future__ import annotations
+
+from typing import Mapping, Optional, Tuple
+
+import torch
+from torch import Tensor, nn
+
+from . import ops
+
+
+class RingMask:
+    """Which cache rows the current frame may attend to, described by reference to the cache
+    state instead of a materialised mask: row ``j`` is visible iff it is in the tail or lies in
+    a written ring slot other than the one the current frame replaces on a persisting frame
+    (``src/model/kv_cache.py:141-143``)."""
+
+    __slots__ = ("kv", "written", "t_pos", "L", "tpf", "dilation")
+
+    def __init__(self, kv: Tensor, written: Tensor, t_pos: Tensor, L: int, tpf: int, dilation: int):
+        self.kv, self.written, self.t_pos = kv, written, t_pos
+        self.L, self.tpf, self.dilation = L, tpf, dilation
+
+    def dense(self) -> Tensor:
+        """The equivalent bool ``[L+T]`` mask (debugging aid; runs small device ops)."""
+        n = self.L // self.tpf
+        t = self.t_pos.reshape(-1)[0]
+        slot = torch.div(t + (self.dilation - 1), self.dilation, rounding_mode="floor") % (n // self.dilation)
+        hide = (t % self.dilation) == 0
+        rows = torch.arange(self.L + self.tpf, device=self.written.device)
+        in_slot = (rows >= slot * self.tpf) & (rows < (slot + 1) * self.tpf)
+        return self.written & ~(in_slot & hide)
+
+
+class LayerKVCache(nn.Module):
+    """One layer's ring: ``L`` history rows in ``L/T`` frame slots plus a ``T``-row tail that
+    always holds the current frame."""
+
+    def __init__(self, B: int, H: int, L: int, Dh: int, dtype: torch.dtype, tokens_per_frame: int,
+                 pinned_dilation: int = 1):
+        super().__init__()
+        T = tokens_per_frame
+        if L % T != 0 or (L // T) % pinned_dilation != 0:
+            raise AssertionError("L must be a multiple of tokens_per_frame and L/T of pinned_dilation")
+        self.tpf = T
+        self.L = L
+        self.capacity = L + T
+        self.pinned_dilation = pinned_dilation
+        self.num_buckets = (L // T) // pinned_dilation
+        self.check_inputs = True  # eager-mode sanity checks like the reference's (they sync)
+
+        self.register_buffer("kv", torch.zeros(2, B, H, self.capacity, Dh, dtype=dtype), persistent=False)
+        written = torch.zeros(self.capacity, dtype=torch.bool)
+        written[L:] = True
+        self.register_buffer("written", written, persistent=False)
+        offsets = torch.arange(T, dtype=torch.long)
+        self.register_buffer("frame_offsets", offsets, persistent=False)
+        self.register_buffer("current_idx", offsets + L, persistent=False)
+
+    def reset(self) -> None:
+        self.kv.zero_()
+        self.written.zero_()
+        self.written[self.L:].fill_(True)
+
+    # -- input checks of the reference's eager path (src/model/kv_cache.py:112-124) ------------
+    def _check(self, k: Tensor, pos_ids: Mapping[str, Tensor]) -> None:
+        t_pos = pos_ids["t_pos"]
+        ops._need_device(k, self.kv, t_pos)
+        if k.size(2) != self.tpf:
+            raise RuntimeError("KV cache expects exactly one frame per upsert")
+        if tuple(t_pos.shape) != (k.size(0), self.tpf):
+            raise RuntimeError("t_pos must be [B, T]")
+        if self.check_inputs and not torch.compiler.is_compiling() and not torch.cuda.is_current_stream_capturing():
+            if not bool((t_pos >= 0).all().item()):
+                raise RuntimeError("t_pos must be non-negative during inference")
+            if not bool((t_pos == t_pos[:, :1]).all().item()):
+                raise RuntimeError("t_pos must be constant within frame")
+
+    def _mask(self, pos_ids: Mapping[str, Tensor]) -> RingMask:
+        return RingMask(self.kv, self.written, pos_ids["t_pos"], self.L, self.tpf, self.pinned_dilation)
+
+    def upsert_kv(self, k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor], is_frozen: bool):
+        """Store already-rotated ``k`` and ``v`` ``[B,H,T,Dh]`` (no stacking copy)."""
+        self._check(k, pos_ids)
+        ops.rope_kv_store(None, k, v, pos_ids, None, None, 1, 1, self.kv, self.written, self.L,
+                          self.pinned_dilation, is_frozen)
+        return self.kv[0], self.kv[1], self._mask(pos_ids)
+
+    def upsert(self, kv: Tensor, pos_ids: Mapping[str, Tensor], is_frozen: bool):
+        """Reference signature: ``kv`` is ``[2,B,H,T,Dh]`` (``src/model/kv_cache.py:104``)."""
+        return self.upsert_kv(kv[0], kv[1], pos_ids, is_frozen)
+
+    def rope_upsert(self, q: Tensor, k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor], rope,
+                    is_frozen: bool):
+        """Fused path used by the attention module: rotate q and k with ``rope``'s tables, store
+        k/v, return ``(RoPE(q), k_all, v_all, mask)`` from a single kernel launch."""
+        self._check(k, pos_ids)
+        q_rot = ops.rope_kv_store(q, k, v, pos_ids, rope.cos, rope.sin, rope.height, rope.width,
+                                  self.kv, self.written, self.L, self.pinned_dilation, is_frozen)
+        return q_rot, self.kv[0], self.kv[1], self._mask(pos_ids)
+
+
+class StaticKVCache(nn.Module):
+    """Per-layer rings with local/global windows chosen as in ``src/model/kv_cache.py:157-181``."""
+
+    def __init__(self, config, batch_size: int, dtype: torch.dtype):
+        super().__init__()
+        self.tpf = config.tokens_per_frame
+        period = config.global_attn_period
+        off = getattr(config, "global_attn_offset", 0) % period
+        n_kv = getattr(config, "n_kv_heads", config.n_heads)
+        d_head = config.d_model // config.n_heads
+        layers = []
+        for idx in range(config.n_layers):
+            is_global = (idx - off) % period == 0
+            frames = config.global_window if is_global else config.local_window
+            dilation = config.global_pinned_dilation if is_global else 1
+            layers.append(LayerKVCache(batch_size, n_kv, frames * self.tpf, d_head, dtype, self.tpf, dilation))
+        self.layers = nn.ModuleList(layers)
+        self._is_frozen = True
+
+    def reset(self) -> None:
+        for layer in self.layers:
+            layer.reset()
+        self._is_frozen = True
+
+    def set_frozen(self, is_frozen: bool) -> None:
+        self._is_frozen = is_frozen
+
+    def upsert(self, k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor], layer: int):
+        return self.layers[layer].upsert_kv(k, v, pos_ids, self._is_frozen)
+
+    def rope_upsert(self, q: Tensor, k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor], rope, layer: int):
+        return self.layers[layer].rope_upsert(q, k, v, pos_ids, rope, self._is_frozen)

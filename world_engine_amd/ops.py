@@ -1,0 +1,232 @@
+"""Python entry points of the HIP kernels (thin wrappers over the C ABI, no fallbacks).
+
+Every function enqueues on the calling thread's current torch stream and returns at once; no
+host synchronisation happens here, so calls can be captured into a HIP graph.  Tensors must live
+on a ROCm device; anything else raises.
+"""
+from __future__ import annotations
+
+import math
+from typing import Mapping, Optional, Tuple
+
+import torch
+
+from . import _capi
+
+Tensor = torch.Tensor
+
+_DTYPE_CODE = {torch.bfloat16: _capi.WE_DTYPE_BF16, torch.float16: _capi.WE_DTYPE_F16,
+               torch.float32: _capi.WE_DTYPE_F32}
+
+
+def _dtype_code(t: Tensor) -> int:
+    try:
+        return _DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise RuntimeError(f"unsupported element type {t.dtype}") from None
+
+
+def _need_device(*tensors: Tensor) -> torch.device:
+    dev = tensors[0].device
+    for t in tensors:
+        if t is None:
+            continue
+        if t.device.type != "cuda":
+            raise RuntimeError("world_engine_amd kernels run on a ROCm GPU only; got a tensor on "
+                               f"{t.device} (there is no CPU path)")
+        if t.device != dev:
+            raise RuntimeError("all tensors must be on the same device")
+    return dev
+
+
+def _stream_ptr(dev: torch.device) -> int:
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+def _bhtd_strides(t: Tensor, what: str):
+    if t.dim() != 4 or t.stride(3) != 1:
+        raise RuntimeError(f"{what} must be [B, H, T, Dh] with a contiguous last dimension")
+    return _capi.i64x3(t.stride(0), t.stride(1), t.stride(2))
+
+
+def _pos_triplet(pos_ids: Mapping[str, Tensor], B: int, T: int, need_yx: bool):
+    """Returns (t_pos, y_pos, x_pos, row_stride); y/x are None when not needed."""
+    t_pos = pos_ids["t_pos"]
+    if tuple(t_pos.shape) != (B, T):
+        raise RuntimeError("t_pos must be [B, T]")
+    if t_pos.dtype != torch.long:
+        raise RuntimeError("position ids must be int64")
+    if not need_yx:
+        if t_pos.stride(1) != 1 and T > 1:
+            t_pos = t_pos.contiguous()
+        return t_pos, None, None, t_pos.stride(0)
+    y_pos, x_pos = pos_ids["y_pos"], pos_ids["x_pos"]
+    for p in (y_pos, x_pos):
+        if tuple(p.shape) != (B, T) or p.dtype != torch.long:
+            raise RuntimeError("y_pos / x_pos must be int64 [B, T]")
+    same = all(p.stride(1) == 1 and p.stride(0) == t_pos.stride(0) for p in (t_pos, y_pos, x_pos))
+    if not same:
+        t_pos, y_pos, x_pos = (p.contiguous() for p in (t_pos, y_pos, x_pos))
+    return t_pos, y_pos, x_pos, t_pos.stride(0)
+
+
+def rope_kv_store(q: Optional[Tensor], k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor],
+                  cos_table: Optional[Tensor], sin_table: Optional[Tensor],
+                  grid_h: int, grid_w: int, kv: Tensor, written: Tensor, L: int, dilation: int,
+                  is_frozen: bool) -> Optional[Tensor]:
+    """Fused RoPE(q), RoPE(k) + tail / ring-slot store of (k, v) + ``written`` update.
+
+    Replaces ``src/model/attn.py:110`` and ``src/model/kv_cache.py:191-193,126-151`` of the
+    reference for one frame.  ``kv`` ``[2,B,Hkv,L+T,Dh]`` and ``written`` ``[L+T]`` are mutated
+    in place.  With ``cos_table is None`` nothing is rotated (k already rotated by the caller).
+    Returns RoPE(q) (contiguous ``[B,H,T,Dh]``) or ``None`` when ``q`` is ``None``.
+    """
+    dev = _need_device(k, v, kv, written, q, cos_table, sin_table, pos_ids["t_pos"])
+    if k.dim() != 4 or k.shape != v.shape:
+        raise RuntimeError("k and v must both be [B, Hkv, T, Dh]")
+    B, Hkv, T, Dh = k.shape
+    if k.dtype != kv.dtype or v.dtype != kv.dtype or (q is not None and q.dtype != kv.dtype):
+        raise RuntimeError("q/k/v must have the cache's element type")
+    if kv.dim() != 5 or tuple(kv.shape) != (2, B, Hkv, L + T, Dh) or not kv.is_contiguous():
+        raise RuntimeError("kv must be a contiguous [2, B, Hkv, L+T, Dh] buffer; "
+                           "KV cache expects exactly one frame per upsert")
+    if written.dtype != torch.bool or written.numel() != L + T or not written.is_contiguous():
+        raise RuntimeError("written must be a contiguous bool [L+T] tensor")
+    H = Hkv
+    q_out = None
+    if q is not None:
+        if q.dim() != 4 or q.shape[0] != B or q.shape[2] != T or q.shape[3] != Dh:
+            raise RuntimeError("q must be [B, H, T, Dh] matching k")
+        H = q.shape[1]
+        q_out = torch.empty((B, H, T, Dh), dtype=q.dtype, device=dev)
+    rotate = cos_table is not None
+    if rotate:
+        if (cos_table.dtype != torch.float32 or sin_table.dtype != torch.float32
+                or cos_table.shape != sin_table.shape or cos_table.dim() != 2
+                or cos_table.shape[1] != Dh // 2
+                or not cos_table.is_contiguous() or not sin_table.is_contiguous()):
+            raise RuntimeError("cos/sin tables must be contiguous fp32 [rows, Dh/2]")
+    t_pos, y_pos, x_pos, ps = _pos_triplet(pos_ids, B, T, rotate)
+    code = _capi.lib().we_rope_kv_store(
+        q.data_ptr() if q is not None else None, k.data_ptr(), v.data_ptr(),
+        _bhtd_strides(q, "q") if q is not None else None, _bhtd_strides(k, "k"), _bhtd_strides(v, "v"),
+        q_out.data_ptr() if q_out is not None else None,
+        cos_table.data_ptr() if rotate else None, sin_table.data_ptr() if rotate else None,
+        cos_table.shape[0] if rotate else 0,
+        t_pos.data_ptr(), y_pos.data_ptr() if rotate else None, x_pos.data_ptr() if rotate else None,
+        ps, grid_h, grid_w, kv.data_ptr(), written.data_ptr(),
+        B, H, Hkv, T, Dh, L, dilation, int(bool(is_frozen)), _dtype_code(kv), _stream_ptr(dev))
+    _capi.check(code, "we_rope_kv_store")
+    return q_out
+
+
+def rope_apply(x: Tensor, pos_ids: Mapping[str, Tensor], cos_table: Tensor, sin_table: Tensor,
+               grid_h: int, grid_w: int) -> Tensor:
+    """Stand-alone RoPE of one ``[B,H,T,Dh]`` tensor (``src/model/attn.py:33-40``)."""
+    dev = _need_device(x, cos_table, sin_table, pos_ids["t_pos"])
+    if x.dim() != 4:
+        raise RuntimeError("x must be [B, H, T, Dh]")
+    B, H, T, Dh = x.shape
+    if cos_table.dtype != torch.float32 or sin_table.dtype != torch.float32:
+        raise RuntimeError("cos/sin tables must be fp32")
+    if cos_table.shape != sin_table.shape or cos_table.dim() != 2 or cos_table.shape[1] != Dh // 2:
+        raise RuntimeError("cos/sin tables must be [rows, Dh/2]")
+    t_pos, y_pos, x_pos, ps = _pos_triplet(pos_ids, B, T, True)
+    out = torch.empty((B, H, T, Dh), dtype=x.dtype, device=dev)
+    code = _capi.lib().we_rope_apply(
+        x.data_ptr(), _bhtd_strides(x, "x"), out.data_ptr(),
+        cos_table.contiguous().data_ptr(), sin_table.contiguous().data_ptr(), cos_table.shape[0],
+        t_pos.data_ptr(), y_pos.data_ptr(), x_pos.data_ptr(), ps, grid_h, grid_w,
+        B, H, T, Dh, _dtype_code(x), _stream_ptr(dev))
+    _capi.check(code, "we_rope_apply")
+    return out
+
+
+def attn_auto_splits(B: int, H: int, Hkv: int, T: int, Dh: int, L: int) -> int:
+    return int(_capi.lib().we_attn_auto_splits(B, H, Hkv, T, Dh, L))
+
+
+def attn_workspace_bytes(B: int, H: int, T: int, Dh: int, n_splits: int) -> int:
+    return int(_capi.lib().we_attn_workspace_bytes(B, H, T, Dh, n_splits))
+
+
+def attn_ring(q: Tensor, kv: Tensor, written: Tensor, t_pos: Tensor, L: int, dilation: int,
+              scale: Optional[float] = None, n_splits: int = 0, q_tile: int = 0,
+              out: Optional[Tensor] = None, workspace: Optional[Tensor] = None,
+              token_major_out: bool = True) -> Tensor:
+    """Attention of one frame's queries over the visible part of the ring buffer.
+
+    Replaces ``make_block_mask`` + ``flex_attention`` (``src/model/kv_cache.py:141-144``,
+    ``src/model/attn.py:116``).  ``q`` ``[B,H,T,Dh]`` (any batch/head/token strides), ``kv``
+    ``[2,B,Hkv,L+T,Dh]``, ``written`` ``[L+T]`` bool, ``t_pos`` int64 with the frame index at
+    element 0.  Returns ``[B,H,T,Dh]``; with ``token_major_out`` its memory is ``[B,T,H,Dh]`` so
+    that ``y.transpose(1, 2).reshape(B, T, H*Dh)`` is a view (``src/patch_model.py:139``).
+    """
+    dev = _need_device(q, kv, written, t_pos)
+    if q.dim() != 4:
+        raise RuntimeError("q must be [B, H, T, Dh]")
+    B, H, T, Dh = q.shape
+    if kv.dim() != 5 or kv.shape[0] != 2 or kv.shape[1] != B or kv.shape[3] != L + T or kv.shape[4] != Dh:
+        raise RuntimeError("kv must be [2, B, Hkv, L+T, Dh] matching q")
+    if not kv.is_contiguous() or kv.dtype != q.dtype:
+        raise RuntimeError("kv must be contiguous and of q's element type")
+    Hkv = kv.shape[2]
+    if written.dtype != torch.bool or written.numel() != L + T or not written.is_contiguous():
+        raise RuntimeError("written must be a contiguous bool [L+T] tensor")
+    if t_pos.dtype != torch.long or t_pos.numel() < 1:
+        raise RuntimeError("t_pos must be a non-empty int64 tensor")
+    scale = 1.0 / math.sqrt(Dh) if scale is None else float(scale)
+    lib = _capi.lib()
+    if n_splits == 0:
+        n_eff = int(lib.we_attn_auto_splits(B, H, Hkv, T, Dh, L))
+    else:
+        n_eff = n_splits
+    ws_bytes = int(lib.we_attn_workspace_bytes(B, H, T, Dh, n_eff))
+    if ws_bytes and (workspace is None or workspace.numel() * workspace.element_size() < ws_bytes):
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    if out is None:
+        if token_major_out:
+            out = torch.empty((B, T, H, Dh), dtype=q.dtype, device=dev).transpose(1, 2)
+        else:
+            out = torch.empty((B, H, T, Dh), dtype=q.dtype, device=dev)
+    elif tuple(out.shape) != (B, H, T, Dh) or out.dtype != q.dtype or out.device != dev:
+        raise RuntimeError("out must be [B, H, T, Dh] of q's element type on q's device")
+    code = lib.we_attn_ring_fwd(
+        q.data_ptr(), _bhtd_strides(q, "q"), kv.data_ptr(), written.data_ptr(), t_pos.data_ptr(),
+        out.data_ptr(), _bhtd_strides(out, "out"),
+        workspace.data_ptr() if ws_bytes else None,
+        workspace.numel() * workspace.element_size() if ws_bytes else 0,
+        B, H, Hkv, T, Dh, L, dilation, scale, n_eff, q_tile, _dtype_code(q), _stream_ptr(dev))
+    _capi.check(code, "we_attn_ring_fwd")
+    return out
+
+
+# --------------------------------------------------------------------------------------------
+# torch.library registration: opaque ops that survive torch.compile(fullgraph=True), the way the
+# reference wraps its one native kernel (src/quantize.py:17-42).
+# --------------------------------------------------------------------------------------------
+@torch.library.custom_op("world_engine_amd::rope_kv_store", mutates_args=("kv", "written"))
+def rope_kv_store_op(q: Tensor, k: Tensor, v: Tensor, t_pos: Tensor, y_pos: Tensor, x_pos: Tensor,
+                     cos_table: Tensor, sin_table: Tensor, grid_h: int, grid_w: int,
+                     kv: Tensor, written: Tensor, L: int, dilation: int, is_frozen: bool) -> Tensor:
+    pos = {"t_pos": t_pos, "y_pos": y_pos, "x_pos": x_pos}
+    return rope_kv_store(q, k, v, pos, cos_table, sin_table, grid_h, grid_w, kv, written, L,
+                         dilation, is_frozen)
+
+
+@rope_kv_store_op.register_fake
+def _rope_kv_store_fake(q, k, v, t_pos, y_pos, x_pos, cos_table, sin_table, grid_h, grid_w,
+                        kv, written, L, dilation, is_frozen):
+    return q.new_empty(q.shape)
+
+
+@torch.library.custom_op("world_engine_amd::attn_ring", mutates_args=())
+def attn_ring_op(q: Tensor, kv: Tensor, written: Tensor, t_pos: Tensor, L: int, dilation: int,
+                 scale: float) -> Tensor:
+    return attn_ring(q, kv, written, t_pos, L, dilation, scale)
+
+
+@attn_ring_op.register_fake
+def _attn_ring_fake(q, kv, written, t_pos, L, dilation, scale):
+    B, H, T, Dh = q.shape
+    return q.new_empty((B, T, H, Dh)).transpose(1, 2)
