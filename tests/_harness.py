@@ -82,19 +82,24 @@ class Pair:
     def assert_state_equal(self, layer=0, what=""):
         o, h = self.oracle.layers[layer], self.hip.layers[layer]
         assert torch.equal(h.written.cpu(), o.written), f"written differs {what}"
-        hk = h.kv.cpu()
-        if not torch.equal(hk.view(torch.uint8), o.kv.view(torch.uint8)):
-            diff = (hk.float() != o.kv.float()).nonzero()
-            raise AssertionError(f"kv buffer differs {what}: {diff.shape[0]} elements, first {diff[0].tolist()}")
+        assert_bits_equal(h.kv, o.kv, f"kv buffer {what}")
 
     def attend(self, q_h, ring, **kw):
         return ops.attn_ring(q_h, ring.kv, ring.written, ring.t_pos, ring.L, ring.dilation, **kw)
 
 
 def assert_bits_equal(a: torch.Tensor, b: torch.Tensor, what=""):
+    """Bit-for-bit equality.  NaNs only have to be NaN on both sides: torch's own fp32->bf16
+    conversions disagree on the NaN bit pattern (0x7FC0 scalar, 0xFFFF vectorised)."""
     a, b = a.cpu().contiguous(), b.cpu().contiguous()
     assert a.shape == b.shape and a.dtype == b.dtype, what
-    assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), f"bit mismatch: {what}"
+    if torch.equal(a.view(torch.uint8), b.view(torch.uint8)):
+        return
+    ib = {1: torch.uint8, 2: torch.int16, 4: torch.int32}[a.element_size()]
+    bad = (a.view(ib) != b.view(ib)) & ~(a.isnan() & b.isnan())
+    if bad.any():
+        idx = bad.nonzero()
+        raise AssertionError(f"bit mismatch: {what}: {idx.shape[0]} elements, first at {idx[0].tolist()}")
 
 
 def assert_attn_close(out_hip: torch.Tensor, ref32: torch.Tensor, what=""):

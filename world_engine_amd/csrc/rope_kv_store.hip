@@ -14,6 +14,10 @@
 #include "we_common.h"
 #include "we_kernels.h"
 
+// The rotation must round each product and the sum separately, like eager fp32 tensor ops;
+// hipcc's default would contract them into fused multiply-adds.
+#pragma clang fp contract(off)
+
 namespace we {
 
 struct Bf16Tag {
@@ -132,8 +136,10 @@ __global__ void __launch_bounds__(256) rope_kv_store_kernel(StoreParams p) {
       const float x1 = Tag::to_f32(in.e[2 * i + 1]);
       // y0 = x0*cos - x1*sin ; y1 = x1*cos + x0*sin with every product and the sum rounded
       // separately (no fused multiply-add), as eager fp32 tensor ops do (attn.py:38-39).
-      const float y0 = __fsub_rn(__fmul_rn(x0, c[i]), __fmul_rn(x1, s[i]));
-      const float y1 = __fadd_rn(__fmul_rn(x1, c[i]), __fmul_rn(x0, s[i]));
+      // (plain operators: the contract(off) pragma above governs them, not inlined intrinsics)
+      const float p0 = x0 * c[i], p1 = x1 * s[i], p2 = x1 * c[i], p3 = x0 * s[i];
+      const float y0 = p0 - p1;
+      const float y1 = p2 + p3;
       lo.e[i] = Tag::from_f32(y0);
       hi.e[i] = Tag::from_f32(y1);
     }
