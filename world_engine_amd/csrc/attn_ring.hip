@@ -18,7 +18,8 @@
 //                                 row-major V tile (the LDS transposing read of gfx950),
 //                                 B = P^T: the S^T accumulators already have the B-operand
 //                                 layout, so P never leaves registers.
-// K/V tiles go HBM -> registers -> LDS, double buffered, one barrier per tile.
+// K/V tiles go HBM -> registers -> LDS (double buffered, one barrier per tile); the global
+// loads of tile i+1 are in flight while tile i is being computed.
 // Workgroup ids are laid out so that the workgroups sharing one K/V stream (query tiles and
 // grouped query heads) run on the same XCD and hit in its L2.
 //
@@ -148,26 +149,27 @@ __global__ void __launch_bounds__(256, NQB == 1 ? 2 : 1) attn_ring_kernel(AttnPa
       reinterpret_cast<const uint16_t*>(p.kv) + ((int64_t)b * p.Hkv + hkv) * cap * DH;
   const uint16_t* vbase = kbase + (int64_t)p.B * p.Hkv * cap * DH;
 
-  uint4 kreg[CPT], vreg[CPT];
-  auto load_tile = [&](int ti) {
+  // One tile in flight: global -> registers (issued a whole compute phase before use) -> LDS.
+  u32x4_t kreg[CPT], vreg[CPT];
+  const int ld_r = tid / CPR, ld_c8 = tid % CPR;  // chunk c = tid + 256*i -> row ld_r + i*(256/CPR)
+  auto load_tile = [&](int ti) __attribute__((always_inline)) {
     const int sidx = ti / tps;
     const int64_t row0 = (int64_t)vis[sidx] * p.T + (int64_t)(ti - sidx * tps) * BN;
+    const uint16_t* kp = kbase + (row0 + ld_r) * DH + ld_c8 * 8;
+    const uint16_t* vp = vbase + (row0 + ld_r) * DH + ld_c8 * 8;
 #pragma unroll
     for (int i = 0; i < CPT; ++i) {
-      const int c = tid + 256 * i;
-      const int r = c / CPR, c8 = c % CPR;
-      const int64_t off = (row0 + r) * DH + c8 * 8;
-      kreg[i] = *reinterpret_cast<const uint4*>(kbase + off);
-      vreg[i] = *reinterpret_cast<const uint4*>(vbase + off);
+      kreg[i] = *reinterpret_cast<const u32x4_t*>(kp + (int64_t)i * (256 / CPR) * DH);
+      vreg[i] = *reinterpret_cast<const u32x4_t*>(vp + (int64_t)i * (256 / CPR) * DH);
     }
   };
-  auto store_tile = [&](int buf) {
+  auto store_tile = [&](int buf) __attribute__((always_inline)) {
+    uint16_t* kd = lds_k + buf * BN * KSTR + ld_r * KSTR + ld_c8 * 8;
+    uint16_t* vd = lds_v + buf * BN * VSTR + ld_r * VSTR + ld_c8 * 8;
 #pragma unroll
     for (int i = 0; i < CPT; ++i) {
-      const int c = tid + 256 * i;
-      const int r = c / CPR, c8 = c % CPR;
-      *reinterpret_cast<uint4*>(lds_k + buf * BN * KSTR + r * KSTR + c8 * 8) = kreg[i];
-      *reinterpret_cast<uint4*>(lds_v + buf * BN * VSTR + r * VSTR + c8 * 8) = vreg[i];
+      *reinterpret_cast<u32x4_t*>(kd + i * (256 / CPR) * KSTR) = kreg[i];
+      *reinterpret_cast<u32x4_t*>(vd + i * (256 / CPR) * VSTR) = vreg[i];
     }
   };
 
@@ -183,12 +185,7 @@ __global__ void __launch_bounds__(256, NQB == 1 ? 2 : 1) attn_ring_kernel(AttnPa
       for (int i = 0; i < 16; ++i) o[qb][db][i] = 0.f;
   }
 
-  if (ntile > 0) {
-    load_tile(t_begin);
-    store_tile(0);
-    if (ntile > 1) load_tile(t_begin + 1);
-  }
-  __syncthreads();
+  if (ntile > 0) load_tile(t_begin);
 
   const float c2 = p.scale_log2;
   // per-lane offsets of the fragment reads
@@ -196,7 +193,12 @@ __global__ void __launch_bounds__(256, NQB == 1 ? 2 : 1) attn_ring_kernel(AttnPa
   const int v_off = (4 * hh + ((lane & 15) >> 2)) * VSTR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
   for (int it = 0; it < ntile; ++it) {
+    // Stage tile `it` into buffer it&1.  Every wave finished reading that buffer (tile it-2)
+    // before it passed the previous iteration's barrier, so one barrier per tile suffices.
     const int buf = it & 1;
+    store_tile(buf);
+    __syncthreads();
+    if (it + 1 < ntile) load_tile(t_begin + it + 1);
     const uint16_t* kt = lds_k + buf * BN * KSTR + k_off;
     const uint16_t* vt = lds_v + buf * BN * VSTR + v_off;
 
@@ -270,10 +272,6 @@ __global__ void __launch_bounds__(256, NQB == 1 ? 2 : 1) attn_ring_kernel(AttnPa
       }
     }
 
-    // ---- stage the next tile, fetch the one after ----
-    if (it + 1 < ntile) store_tile(buf ^ 1);
-    if (it + 2 < ntile) load_tile(t_begin + it + 2);
-    __syncthreads();
   }
 
   // ---- epilogue ----

@@ -26,21 +26,21 @@ struct AttnPlan {
   int n_splits;
 };
 
-// Pick the query-tile size and the number of context splits so that the grid fills the 256 CUs
-// (two 128-query workgroups or one 256-query workgroup fit per CU) without making a split
-// shorter than two 64-key tiles of the steady-state context.
+// Pick the query-tile size and the number of context splits.  128-query workgroups (two fit per
+// CU, so softmax VALU work of one overlaps MFMA work of the other) measured faster than
+// 256-query ones at every benchmark shape.  Splits are added until the grid has one workgroup
+// per CU, but never so many that a split holds fewer than two 64-key tiles of the steady-state
+// context.
 AttnPlan plan_attn(int B, int H, int T, int64_t L, int n_splits, int variant) {
   AttnPlan pl;
-  const int64_t wg256 = (int64_t)B * H * ((T + 255) / 256);
-  pl.variant = variant ? variant : ((wg256 >= 256 && T >= 256) ? 2 : 1);
+  pl.variant = variant ? variant : 1;
   if (n_splits > 0) {
     pl.n_splits = n_splits;
     return pl;
   }
   const int bm = pl.variant == 2 ? 256 : 128;
   const int64_t base = (int64_t)B * H * ((T + bm - 1) / bm);
-  const int64_t slots_per_cu = pl.variant == 2 ? 1 : 2;
-  const int64_t want = 256 * slots_per_cu;
+  const int64_t want = 256;
   int s = 1;
   if (base < want) {
     s = (int)((want + base - 1) / base);
