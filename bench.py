@@ -175,19 +175,25 @@ def main():
     for _ in range(5):
         attn_only()
     torch.cuda.synchronize()
-    g2 = torch.cuda.CUDAGraph()
-    side2 = torch.cuda.Stream()
-    side2.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.graph(g2, stream=side2):
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    if args.eager:
+        e0.record()
         for _ in range(iters):
             attn_only()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    g2.replay()
-    torch.cuda.synchronize()
-    e0.record()
-    g2.replay()
-    e1.record()
+        e1.record()
+    else:
+        g2 = torch.cuda.CUDAGraph()
+        side2 = torch.cuda.Stream()
+        side2.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.graph(g2, stream=side2):
+            for _ in range(iters):
+                attn_only()
+        torch.cuda.synchronize()
+        g2.replay()
+        torch.cuda.synchronize()
+        e0.record()
+        g2.replay()
+        e1.record()
     torch.cuda.synchronize()
     attn_us = e0.elapsed_time(e1) * 1e3 / iters
     n_vis = L                                        # steady state: n-1 ring slots + the tail

@@ -33,8 +33,12 @@ namespace we {
 
 constexpr int BN = 64;  // keys per tile
 
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+
 struct Bf16Mma {
   typedef bf16x8_t frag_t;
+  typedef __bf16 elem_t;
   __device__ static __forceinline__ f32x16_t mma(frag_t a, frag_t b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
@@ -45,9 +49,22 @@ struct Bf16Mma {
     r[4] = (__bf16)v4; r[5] = (__bf16)v5; r[6] = (__bf16)v6; r[7] = (__bf16)v7;
     return r;
   }
+  // acc + the two elements of one packed register (v_dot2c_f32_bf16 with a (1, 1) operand)
+  __device__ static __forceinline__ float add_pair(float acc, frag_t f, int pair) {
+    const bf16x2_t ones = {(__bf16)1.0f, (__bf16)1.0f};
+    const bf16x2_t v = {f[2 * pair], f[2 * pair + 1]};
+    return __builtin_amdgcn_fdot2_f32_bf16(v, ones, acc, false);
+  }
+  // smallest bf16-representable value >= x (x finite)
+  __device__ static __forceinline__ float round_up(float x) {
+    uint32_t u = __float_as_uint(x);
+    u = (x >= 0.f) ? (u + 0xffffu) & 0xffff0000u : (u & 0xffff0000u);
+    return __uint_as_float(u);
+  }
 };
 struct F16Mma {
   typedef f16x8_t frag_t;
+  typedef _Float16 elem_t;
   __device__ static __forceinline__ f32x16_t mma(frag_t a, frag_t b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
@@ -56,6 +73,22 @@ struct F16Mma {
     frag_t r;
     r[0] = (_Float16)v0; r[1] = (_Float16)v1; r[2] = (_Float16)v2; r[3] = (_Float16)v3;
     r[4] = (_Float16)v4; r[5] = (_Float16)v5; r[6] = (_Float16)v6; r[7] = (_Float16)v7;
+    return r;
+  }
+  __device__ static __forceinline__ float add_pair(float acc, frag_t f, int pair) {
+    const f16x2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
+    const f16x2_t v = {f[2 * pair], f[2 * pair + 1]};
+    return __builtin_amdgcn_fdot2(v, ones, acc, false);
+  }
+  // smallest f16-representable value >= x (|x| well inside the f16 range)
+  __device__ static __forceinline__ float round_up(float x) {
+    const _Float16 h = (_Float16)x;  // nearest
+    float r = (float)h;
+    if (r < x) {
+      uint16_t b = __builtin_bit_cast(uint16_t, h);
+      b = (r >= 0.f) ? (uint16_t)(b + 1) : (uint16_t)(b - 1);
+      r = (float)__builtin_bit_cast(_Float16, b);
+    }
     return r;
   }
 };
@@ -129,7 +162,9 @@ __global__ void __launch_bounds__(256, NQB == 1 ? 2 : 1) attn_ring_kernel(AttnPa
   const int t_end = (int)((int64_t)(split + 1) * nt / p.n_splits);
   const int ntile = t_end - t_begin;
 
-  // ---- Q fragments stay in registers for the whole kernel ----
+  // ---- Q fragments stay in registers for the whole kernel, pre-multiplied by scale*log2(e) so
+  // the matrix product yields base-2 logits directly ----
+  const float c2 = p.scale_log2;
   frag_t qf[NQB][KS];
   int qrow[NQB];
   {
@@ -140,7 +175,11 @@ __global__ void __launch_bounds__(256, NQB == 1 ? 2 : 1) attn_ring_kernel(AttnPa
       const int qr = qrow[qb] < p.T ? qrow[qb] : p.T - 1;
       const uint16_t* src = qbase + (int64_t)qr * p.qs_t + hh * 8;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) qf[qb][ks] = *reinterpret_cast<const frag_t*>(src + ks * 16);
+      for (int ks = 0; ks < KS; ++ks) {
+        const frag_t raw = *reinterpret_cast<const frag_t*>(src + ks * 16);
+        qf[qb][ks] = M::pack8((float)raw[0] * c2, (float)raw[1] * c2, (float)raw[2] * c2, (float)raw[3] * c2,
+                              (float)raw[4] * c2, (float)raw[5] * c2, (float)raw[6] * c2, (float)raw[7] * c2);
+      }
     }
   }
 
@@ -149,35 +188,69 @@ __global__ void __launch_bounds__(256, NQB == 1 ? 2 : 1) attn_ring_kernel(AttnPa
       reinterpret_cast<const uint16_t*>(p.kv) + ((int64_t)b * p.Hkv + hkv) * cap * DH;
   const uint16_t* vbase = kbase + (int64_t)p.B * p.Hkv * cap * DH;
 
-  // One tile in flight: global -> registers (issued a whole compute phase before use) -> LDS.
+  // ---- software pipeline -------------------------------------------------------------------
+  // Iteration `it` holds the logits of tile `it` (s_cur), computes the logits of tile it+1 and
+  // the P*V product of tile it-1 on the matrix cores while the VALU turns s_cur into
+  // probabilities.  LDS: K(it+1) in kb[(it+1)&1], V(it-1) in vb[(it-1)&1]; the stores of K(it+2)
+  // and V(it) go into the two buffers nobody reads during this iteration, so one barrier per
+  // tile is enough.  Global loads run one iteration ahead of their LDS store (K(it+3), V(it+1)).
+  // Tile indices past the end are clamped (the last tile is re-loaded and its logits recomputed
+  // once), which keeps the loop body free of branches.
+  //
+  // The logits leave the matrix cores already shifted by the running reference m_ref: one extra
+  // MFMA per 32-key block multiplies a column of ones (K side) with a fragment holding -m_ref
+  // (Q side; m_ref is kept representable in the element type so the shift is exact).  The VALU
+  // work per element is then exp2, a pack, and half a dot2 for the row sum.  m_ref is raised
+  // only when a row sum shows a probability above 2^8 (then that tile is redone exactly); being
+  // larger than the true running max is never needed for fp32 accumulators.
   u32x4_t kreg[CPT], vreg[CPT];
   const int ld_r = tid / CPR, ld_c8 = tid % CPR;  // chunk c = tid + 256*i -> row ld_r + i*(256/CPR)
-  auto load_tile = [&](int ti) __attribute__((always_inline)) {
-    const int sidx = ti / tps;
-    const int64_t row0 = (int64_t)vis[sidx] * p.T + (int64_t)(ti - sidx * tps) * BN;
-    const uint16_t* kp = kbase + (row0 + ld_r) * DH + ld_c8 * 8;
-    const uint16_t* vp = vbase + (row0 + ld_r) * DH + ld_c8 * 8;
-#pragma unroll
-    for (int i = 0; i < CPT; ++i) {
-      kreg[i] = *reinterpret_cast<const u32x4_t*>(kp + (int64_t)i * (256 / CPR) * DH);
-      vreg[i] = *reinterpret_cast<const u32x4_t*>(vp + (int64_t)i * (256 / CPR) * DH);
+  struct TileWalk {  // position of a load stream in this split's list of visible tiles
+    int sidx, sub, left;
+  };
+  auto walk_init = [&](int ti) __attribute__((always_inline)) {
+    TileWalk w;
+    const int g = t_begin + (ti < ntile ? ti : ntile - 1);
+    w.sidx = g / tps;
+    w.sub = g - w.sidx * tps;
+    w.left = ntile - 1 - (ti < ntile ? ti : ntile - 1);
+    return w;
+  };
+  auto walk_next = [&](TileWalk& w) __attribute__((always_inline)) {
+    if (w.left > 0) {
+      --w.left;
+      if (++w.sub == tps) {
+        w.sub = 0;
+        ++w.sidx;
+      }
     }
   };
-  auto store_tile = [&](int buf) __attribute__((always_inline)) {
-    uint16_t* kd = lds_k + buf * BN * KSTR + ld_r * KSTR + ld_c8 * 8;
-    uint16_t* vd = lds_v + buf * BN * VSTR + ld_r * VSTR + ld_c8 * 8;
-#pragma unroll
-    for (int i = 0; i < CPT; ++i) {
-      *reinterpret_cast<u32x4_t*>(kd + i * (256 / CPR) * KSTR) = kreg[i];
-      *reinterpret_cast<u32x4_t*>(vd + i * (256 / CPR) * VSTR) = vreg[i];
-    }
+  auto tile_ptr = [&](const uint16_t* base, const TileWalk& w) __attribute__((always_inline)) {
+    const int slot = __builtin_amdgcn_readfirstlane(vis[w.sidx]);
+    const int64_t row0 = (int64_t)slot * p.T + (int64_t)w.sub * BN;
+    return base + (row0 + ld_r) * DH + ld_c8 * 8;
   };
+  auto gload = [&](u32x4_t(&r)[CPT], const uint16_t* src) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < CPT; ++i)
+      r[i] = *reinterpret_cast<const u32x4_t*>(src + (int64_t)i * (256 / CPR) * DH);
+  };
+  auto lstore = [&](uint16_t* dst, int stride, const u32x4_t(&r)[CPT]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) *reinterpret_cast<u32x4_t*>(dst + i * (256 / CPR) * stride) = r[i];
+  };
+  uint16_t* const k_st = lds_k + ld_r * KSTR + ld_c8 * 8;  // this thread's staging slots
+  uint16_t* const v_st = lds_v + ld_r * VSTR + ld_c8 * 8;
+  // per-lane offsets of the fragment reads
+  const uint16_t* const k_rd = lds_k + l32 * KSTR + hh * 8;
+  const uint16_t* const v_rd =
+      lds_v + (4 * hh + ((lane & 15) >> 2)) * VSTR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
   f32x16_t o[NQB][DB];
-  float m_run[NQB], l_run[NQB];
+  float m_ref[NQB], l_run[NQB];
 #pragma unroll
   for (int qb = 0; qb < NQB; ++qb) {
-    m_run[qb] = -INFINITY;
+    m_ref[qb] = -INFINITY;
     l_run[qb] = 0.f;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
@@ -185,31 +258,24 @@ __global__ void __launch_bounds__(256, NQB == 1 ? 2 : 1) attn_ring_kernel(AttnPa
       for (int i = 0; i < 16; ++i) o[qb][db][i] = 0.f;
   }
 
-  if (ntile > 0) load_tile(t_begin);
+  const f32x16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  // K-side fragment of the shift product: contraction index 0 is one for every key
+  frag_t ones_frag = __builtin_bit_cast(frag_t, u32x4_t{0u, 0u, 0u, 0u});
+  if (hh == 0) ones_frag[0] = (typename M::elem_t)1.0f;
+  // Q-side fragment: contraction index 0 carries -m_ref of this lane's query
+  frag_t shift[NQB];
+  auto set_shift = [&](int qb) __attribute__((always_inline)) {
+    shift[qb] = __builtin_bit_cast(frag_t, u32x4_t{0u, 0u, 0u, 0u});
+    if (hh == 0) shift[qb][0] = (typename M::elem_t)(-m_ref[qb]);
+  };
 
-  const float c2 = p.scale_log2;
-  // per-lane offsets of the fragment reads
-  const int k_off = l32 * KSTR + hh * 8;
-  const int v_off = (4 * hh + ((lane & 15) >> 2)) * VSTR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-
-  for (int it = 0; it < ntile; ++it) {
-    // Stage tile `it` into buffer it&1.  Every wave finished reading that buffer (tile it-2)
-    // before it passed the previous iteration's barrier, so one barrier per tile suffices.
-    const int buf = it & 1;
-    store_tile(buf);
-    __syncthreads();
-    if (it + 1 < ntile) load_tile(t_begin + it + 1);
-    const uint16_t* kt = lds_k + buf * BN * KSTR + k_off;
-    const uint16_t* vt = lds_v + buf * BN * VSTR + v_off;
-
-    // ---- S^T = K Q^T : two 32-key blocks ----
-    f32x16_t s[NQB][2];
+  // logits of one 64-key tile in LDS buffer `kt`, already minus m_ref when `shifted`
+  auto logits = [&](f32x16_t(&s)[NQB][2], const uint16_t* kt, bool shifted) __attribute__((always_inline)) {
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
       for (int qb = 0; qb < NQB; ++qb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) s[qb][kb][i] = 0.f;
+        s[qb][kb] = shifted ? M::mma(ones_frag, shift[qb], zero16) : zero16;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         const frag_t a = *reinterpret_cast<const frag_t*>(kt + kb * 32 * KSTR + ks * 16);
@@ -217,46 +283,9 @@ __global__ void __launch_bounds__(256, NQB == 1 ? 2 : 1) attn_ring_kernel(AttnPa
         for (int qb = 0; qb < NQB; ++qb) s[qb][kb] = M::mma(a, qf[qb][ks], s[qb][kb]);
       }
     }
-
-    // ---- online softmax; each lane owns one query column ----
-    frag_t pf[NQB][4];
-#pragma unroll
-    for (int qb = 0; qb < NQB; ++qb) {
-      float mx = s[qb][0][0];
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[qb][kb][i]);
-      float lo, up;
-      half_wave_pair(mx, lo, up);
-      mx = fmaxf(lo, up);
-      const float m_new = fmaxf(m_run[qb], mx * c2);
-      const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - m_new);
-      float rs = 0.f;
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qb][kb][i], c2, -m_new));
-          s[qb][kb][i] = e;
-          rs += e;
-        }
-      l_run[qb] = l_run[qb] * alpha + rs;
-      m_run[qb] = m_new;
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) o[qb][db][i] *= alpha;
-#pragma unroll
-      for (int m = 0; m < 4; ++m) {
-        const f32x16_t& sv = s[qb][m >> 1];
-        const int r0 = 8 * (m & 1);
-        pf[qb][m] = M::pack8(sv[r0], sv[r0 + 1], sv[r0 + 2], sv[r0 + 3], sv[r0 + 4], sv[r0 + 5],
-                             sv[r0 + 6], sv[r0 + 7]);
-      }
-    }
-
-    // ---- O^T += V^T P^T : 4 chunks of 16 keys x DB blocks of 32 head-dim rows ----
+  };
+  // O^T += V^T P^T for one 64-key tile in LDS buffer `vt`
+  auto accumulate = [&](const frag_t(&pf)[NQB][4], const uint16_t* vt) __attribute__((always_inline)) {
 #pragma unroll
     for (int m = 0; m < 4; ++m) {
 #pragma unroll
@@ -271,8 +300,154 @@ __global__ void __launch_bounds__(256, NQB == 1 ? 2 : 1) attn_ring_kernel(AttnPa
         for (int qb = 0; qb < NQB; ++qb) o[qb][db] = M::mma(a, pf[qb][m], o[qb][db]);
       }
     }
+  };
+  // probabilities of one tile from its shifted logits: p = 2^s, packed to the element type;
+  // returns this half-wave's share of the row sum (of the rounded values)
+  auto probabilities = [&](frag_t(&pf)[4], const f32x16_t(&s)[2], float sub) __attribute__((always_inline)) {
+    float rs = 0.f;
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const f32x16_t& sv = s[m >> 1];
+      const int r0 = 8 * (m & 1);
+      float e[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) e[j] = __builtin_amdgcn_exp2f(sv[r0 + j] - sub);
+      pf[m] = M::pack8(e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) rs = M::add_pair(rs, pf[m], j);
+    }
+    return rs;
+  };
+  auto tile_max = [&](const f32x16_t(&s)[2]) __attribute__((always_inline)) {
+    float mx = s[0][0];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kb][i]);
+    float lo, up;
+    half_wave_pair(mx, lo, up);
+    return fmaxf(lo, up);
+  };
 
+  if (ntile > 0) {
+    frag_t p_prev[NQB][4];
+    f32x16_t s_cur[NQB][2];
+    {
+      // zero V buffer 1 and P so that the first iteration's product adds exact zeros
+      const u32x4_t z = {0u, 0u, 0u, 0u};
+      for (int i = tid; i < BN * VSTR / 8; i += 256)
+        *reinterpret_cast<u32x4_t*>(lds_v + BN * VSTR + i * 8) = z;
+#pragma unroll
+      for (int qb = 0; qb < NQB; ++qb)
+#pragma unroll
+        for (int m = 0; m < 4; ++m) p_prev[qb][m] = __builtin_bit_cast(frag_t, z);
+    }
+    TileWalk kw = walk_init(0), vw = walk_init(0);
+    gload(kreg, tile_ptr(kbase, kw));  // K(0)
+    walk_next(kw);
+    gload(vreg, tile_ptr(kbase, kw));  // K(1)
+    walk_next(kw);
+    lstore(k_st, KSTR, kreg);
+    lstore(k_st + BN * KSTR, KSTR, vreg);
+    gload(kreg, tile_ptr(kbase, kw));  // K(2)
+    walk_next(kw);
+    gload(vreg, tile_ptr(vbase, vw));  // V(0)
+    walk_next(vw);
+    __syncthreads();
+    // first tile: plain logits, reference = its row max, then shift by hand
+    logits(s_cur, k_rd, false);
+#pragma unroll
+    for (int qb = 0; qb < NQB; ++qb) {
+      m_ref[qb] = M::round_up(tile_max(s_cur[qb]));
+      set_shift(qb);
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s_cur[qb][kb][i] -= m_ref[qb];
+    }
+    __syncthreads();  // K buffer 0 is overwritten by the first iteration
+
+    // A raise decided in iteration it rescales the accumulators after the product of tile it-1
+    // and before that of tile it, i.e. at the top of iteration it+1; with the branch there the
+    // rest of the body stays one basic block for the scheduler to interleave.
+    bool pending = false;
+    float alpha[NQB];
+#pragma unroll
+    for (int qb = 0; qb < NQB; ++qb) alpha[qb] = 1.f;
+    auto rescale = [&]() __attribute__((always_inline)) {
+#pragma unroll
+      for (int qb = 0; qb < NQB; ++qb)
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) o[qb][db][i] *= alpha[qb];
+    };
+
+    for (int it = 0; it < ntile; ++it) {
+      if (pending) rescale();
+      pending = false;
+      const int cur = it & 1, nxt = cur ^ 1;
+      lstore(k_st + cur * BN * KSTR, KSTR, kreg);  // K(it+2)
+      lstore(v_st + cur * BN * VSTR, VSTR, vreg);  // V(it)
+      gload(kreg, tile_ptr(kbase, kw));            // K(it+3)
+      walk_next(kw);
+      gload(vreg, tile_ptr(vbase, vw));            // V(it+1)
+      walk_next(vw);
+
+      // matrix cores: shifted logits of tile it+1
+      f32x16_t s_next[NQB][2];
+      logits(s_next, k_rd + nxt * BN * KSTR, true);
+
+      // VALU: probabilities of tile it
+      frag_t p_cur[NQB][4];
+      float rs[NQB];
+      bool bad = false;
+#pragma unroll
+      for (int qb = 0; qb < NQB; ++qb) {
+        rs[qb] = probabilities(p_cur[qb], s_cur[qb], 0.f);
+        bad = bad || !(rs[qb] <= 256.f);
+      }
+
+      // matrix cores: O += P(it-1) V(it-1)
+      accumulate(p_prev, v_rd + nxt * BN * VSTR);
+
+      if (__ballot(bad) != 0ull) {
+        // Rare: some probability of this tile may exceed 2^8.  Raise the reference of the rows
+        // that need it, redo the tile's probabilities exactly, and re-base the logits of the
+        // next tile, which were produced with the old reference.
+#pragma unroll
+        for (int qb = 0; qb < NQB; ++qb) {
+          const float mx = tile_max(s_cur[qb]);
+          const float m_new = mx > 0.f ? M::round_up(m_ref[qb] + mx) : m_ref[qb];
+          const float delta = m_new - m_ref[qb];
+          alpha[qb] = __builtin_amdgcn_exp2f(-delta);
+          rs[qb] = probabilities(p_cur[qb], s_cur[qb], delta);
+          l_run[qb] *= alpha[qb];
+          m_ref[qb] = m_new;
+          set_shift(qb);
+#pragma unroll
+          for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s_next[qb][kb][i] -= delta;
+        }
+        pending = true;
+      }
+#pragma unroll
+      for (int qb = 0; qb < NQB; ++qb) {
+        l_run[qb] += rs[qb];
+#pragma unroll
+        for (int m = 0; m < 4; ++m) p_prev[qb][m] = p_cur[qb][m];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) s_cur[qb][kb] = s_next[qb][kb];
+      }
+      __syncthreads();
+    }
+    if (pending) rescale();
+    accumulate(p_prev, v_rd + ((ntile - 1) & 1) * BN * VSTR);
   }
+  float m_run[NQB];
+#pragma unroll
+  for (int qb = 0; qb < NQB; ++qb) m_run[qb] = m_ref[qb];
 
   // ---- epilogue ----
   const int64_t rows = (int64_t)p.B * p.H * p.T;
