@@ -25,82 +25,11 @@
 //
 // Roofline: 4*T*N_vis*Dh flops and 4*N_vis*Dh bytes of K/V per (batch, kv head); HBM-bound for
 // 256-query frames (with context splits to fill 256 CUs), MFMA-bound for 1024-query frames.
-#include "we_common.h"
+#include "attn_mma.h"
 #include "we_kernels.h"
 #include "../../include/we_attn.h"
 
 namespace we {
-
-constexpr int BN = 64;  // keys per tile
-
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
-
-struct Bf16Mma {
-  typedef bf16x8_t frag_t;
-  typedef __bf16 elem_t;
-  __device__ static __forceinline__ f32x16_t mma(frag_t a, frag_t b, f32x16_t c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-  }
-  __device__ static __forceinline__ frag_t pack8(float v0, float v1, float v2, float v3, float v4,
-                                                 float v5, float v6, float v7) {
-    frag_t r;
-    r[0] = (__bf16)v0; r[1] = (__bf16)v1; r[2] = (__bf16)v2; r[3] = (__bf16)v3;
-    r[4] = (__bf16)v4; r[5] = (__bf16)v5; r[6] = (__bf16)v6; r[7] = (__bf16)v7;
-    return r;
-  }
-  // acc + the two elements of one packed register (v_dot2c_f32_bf16 with a (1, 1) operand)
-  __device__ static __forceinline__ float add_pair(float acc, frag_t f, int pair) {
-    const bf16x2_t ones = {(__bf16)1.0f, (__bf16)1.0f};
-    const bf16x2_t v = {f[2 * pair], f[2 * pair + 1]};
-    return __builtin_amdgcn_fdot2_f32_bf16(v, ones, acc, false);
-  }
-  // smallest bf16-representable value >= x (x finite)
-  __device__ static __forceinline__ float round_up(float x) {
-    uint32_t u = __float_as_uint(x);
-    u = (x >= 0.f) ? (u + 0xffffu) & 0xffff0000u : (u & 0xffff0000u);
-    return __uint_as_float(u);
-  }
-};
-struct F16Mma {
-  typedef f16x8_t frag_t;
-  typedef _Float16 elem_t;
-  __device__ static __forceinline__ f32x16_t mma(frag_t a, frag_t b, f32x16_t c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-  }
-  __device__ static __forceinline__ frag_t pack8(float v0, float v1, float v2, float v3, float v4,
-                                                 float v5, float v6, float v7) {
-    frag_t r;
-    r[0] = (_Float16)v0; r[1] = (_Float16)v1; r[2] = (_Float16)v2; r[3] = (_Float16)v3;
-    r[4] = (_Float16)v4; r[5] = (_Float16)v5; r[6] = (_Float16)v6; r[7] = (_Float16)v7;
-    return r;
-  }
-  __device__ static __forceinline__ float add_pair(float acc, frag_t f, int pair) {
-    const f16x2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
-    const f16x2_t v = {f[2 * pair], f[2 * pair + 1]};
-    return __builtin_amdgcn_fdot2(v, ones, acc, false);
-  }
-  // smallest f16-representable value >= x (|x| well inside the f16 range)
-  __device__ static __forceinline__ float round_up(float x) {
-    const _Float16 h = (_Float16)x;  // nearest
-    float r = (float)h;
-    if (r < x) {
-      uint16_t b = __builtin_bit_cast(uint16_t, h);
-      b = (r >= 0.f) ? (uint16_t)(b + 1) : (uint16_t)(b - 1);
-      r = (float)__builtin_bit_cast(_Float16, b);
-    }
-    return r;
-  }
-};
-
-// Both half-waves get (lower half's x, upper half's x).
-__device__ __forceinline__ void half_wave_pair(float x, float& lower, float& upper) {
-  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-  lower = __uint_as_float(r[0]);
-  upper = __uint_as_float(r[1]);
-}
-
-typedef __attribute__((address_space(3))) s16x4_t* lds_s16x4_ptr;
 
 template <int DH>
 struct AttnLds {

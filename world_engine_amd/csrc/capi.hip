@@ -38,7 +38,7 @@ AttnPlan plan_attn(int B, int H, int T, int64_t L, int n_splits, int variant) {
     pl.n_splits = n_splits;
     return pl;
   }
-  const int bm = pl.variant == 2 ? 256 : 128;
+  const int bm = (pl.variant == 2 || pl.variant == 4) ? 256 : 128;
   const int64_t base = (int64_t)B * H * ((T + bm - 1) / bm);
   const int64_t want = 256;
   int s = 1;
@@ -162,12 +162,13 @@ int we_attn_ring_fwd(const void* q, const int64_t q_strides[3], const void* kv, 
   if (Dh != 64 && Dh != 128) return WE_ERR_UNSUPPORTED;
   if (T % 64 != 0 || L / T > WE_MAX_SLOTS) return WE_ERR_UNSUPPORTED;
   if (!(scale > 0.f) || n_splits < 0 || n_splits > 64) return WE_ERR_BAD_SHAPE;
-  if (q_tile != 0 && q_tile != 128 && q_tile != 256) return WE_ERR_UNSUPPORTED;
+  if (q_tile != 0 && q_tile != 128 && q_tile != 256 && q_tile != 129 && q_tile != 257) return WE_ERR_UNSUPPORTED;
   if (!aligned16(q) || !aligned16(kv) || !aligned16(out) || !strides_ok(q_strides, dtype) ||
       !strides_ok(out_strides, dtype))
     return WE_ERR_ALIGNMENT;
 
-  const int variant = q_tile == 0 ? 0 : (q_tile == 256 ? 2 : 1);
+  // 128/256: 4-wavefront kernel; 129/257: 8-wavefront LDS-DMA kernel with 128/256 queries
+  const int variant = q_tile == 0 ? 0 : (q_tile == 256 ? 2 : (q_tile == 129 ? 3 : (q_tile == 257 ? 4 : 1)));
   const AttnPlan pl = plan_attn(B, H, T, L, n_splits, variant);
   if (pl.n_splits > 1) {
     if (!workspace || !aligned16(workspace)) return WE_ERR_WORKSPACE;
@@ -185,14 +186,16 @@ int we_attn_ring_fwd(const void* q, const int64_t q_strides[3], const void* kv, 
   p.B = B; p.H = H; p.Hkv = Hkv; p.T = T;
   p.n_slots = (int)(L / T); p.dilation = dilation; p.num_buckets = p.n_slots / dilation;
   p.n_splits = pl.n_splits;
-  const int bm = we::attn_block_m(Dh, pl.variant);
+  const int bm = (pl.variant == 2 || pl.variant == 4) ? 256 : 128;
   p.q_tiles = (T + bm - 1) / bm;
   p.members = (H / Hkv) * p.q_tiles;
   p.unit_splits = B * Hkv * pl.n_splits;
   p.scale_log2 = scale * 1.4426950408889634f;
 
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (we::launch_attn_ring(p, Dh, dtype, pl.variant, st) != hipSuccess) return WE_ERR_LAUNCH;
+  const hipError_t le = pl.variant >= 3 ? we::launch_attn_ring8(p, Dh, dtype, pl.variant == 3 ? 2 : 1, st)
+                                        : we::launch_attn_ring(p, Dh, dtype, pl.variant, st);
+  if (le != hipSuccess) return WE_ERR_LAUNCH;
   if (pl.n_splits > 1 && we::launch_attn_combine(p, Dh, dtype, st) != hipSuccess) return WE_ERR_LAUNCH;
   return WE_OK;
 }

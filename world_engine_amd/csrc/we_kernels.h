@@ -54,6 +54,8 @@ hipError_t launch_rope_kv_store(const StoreParams& p, int dtype, hipStream_t str
 // queries handled by one workgroup of the attention kernel for a head dim / variant
 int attn_block_m(int Dh, int variant);
 hipError_t launch_attn_ring(const AttnParams& p, int Dh, int dtype, int variant, hipStream_t stream);
+// 8-wavefront LDS-DMA kernel: groups = 2 -> 128 queries per workgroup, 1 -> 256
+hipError_t launch_attn_ring8(const AttnParams& p, int Dh, int dtype, int groups, hipStream_t stream);
 hipError_t launch_attn_combine(const AttnParams& p, int Dh, int dtype, hipStream_t stream);
 
 }  // namespace we
