@@ -80,18 +80,36 @@ struct IntC {
   static constexpr int value = V;
 };
 
-template <typename M, int DH, int GROUPS>
+// ---- LDS fragment reads ---------------------------------------------------------------------
+// Left alone, the compiler keeps a single fragment read in flight ahead of the MFMA that needs
+// it, which exposes the full LDS latency on every MFMA.  The hot loop therefore states its reads
+// early in program order, several fragments ahead of their MFMAs, and pins that order with
+// sched_barrier; the reads stay ordinary loads, so the compiler still places the (counted)
+// lgkmcnt waits itself and knows the registers are in flight.
+template <int OFF>
+__device__ __forceinline__ u32x4_t lds_read128(const unsigned char* smem, uint32_t off) {
+  return *reinterpret_cast<const u32x4_t*>(smem + off + OFF);
+}
+template <int OFF>
+__device__ __forceinline__ u32x2_t lds_read_tr(const unsigned char* smem, uint32_t off) {
+  const s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(smem + off + OFF));
+  return __builtin_bit_cast(u32x2_t, v);
+}
+
+template <typename M, int DH, int KSPLIT>
 __global__ void __launch_bounds__(512, 2) attn_ring8_kernel(AttnParams p) {
   typedef typename M::frag_t frag_t;
   typedef Ring8Lds<DH> L;
   constexpr int KS = DH / 16;               // contraction steps of K Q^T
   constexpr int DB = DH / 32;               // 32-row blocks of O^T
-  constexpr int WPG = 8 / GROUPS;           // wavefronts per group
-  constexpr int NST = 4 / GROUPS;           // ring slots per operand and group
-  constexpr int BM = 32 * WPG;              // queries per workgroup
+  constexpr int NV = 2 * DB;                // V^T fragments of one 32-key block
+  constexpr int QW = 8 / KSPLIT;            // wavefronts with distinct query blocks
+  constexpr int BM = 32 * QW;               // queries per workgroup
+  constexpr int NST = 4;                    // ring slots per operand
   constexpr int CPR = L::CPR, ROW_B = L::ROW_B, TILE_B = L::TILE_B;
+  constexpr int KB_B = 32 * ROW_B;          // bytes of one 32-key block of a tile
   constexpr int RPI = 1024 / ROW_B;         // rows moved by one DMA instruction
-  constexpr int NDMA = TILE_B / 1024 / WPG; // DMA instructions per wavefront and tile operand
+  constexpr int NDMA = TILE_B / 1024 / 8;   // DMA instructions per wavefront and tile operand
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   int* vis = reinterpret_cast<int*>(smem + L::MISC_OFF);  // visible slots, then their count
@@ -100,7 +118,8 @@ __global__ void __launch_bounds__(512, 2) attn_ring8_kernel(AttnParams p) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, hh = lane >> 5;
-  const int grp = wave / WPG, wig = wave % WPG;
+  const int qb = wave % QW;   // query block of this wavefront
+  const int hb = wave / QW;   // key block of every tile it handles when KSPLIT == 2 (else 0)
 
   // ---- which (batch, head, query tile, split) this workgroup owns; XCD = blockIdx % 8 ----
   const int xcd = blockIdx.x & 7, jj = blockIdx.x >> 3;
@@ -131,19 +150,31 @@ __global__ void __launch_bounds__(512, 2) attn_ring8_kernel(AttnParams p) {
   }
   __syncthreads();
   const int nvis = __builtin_amdgcn_readfirstlane(vis[WE_MAX_SLOTS + 1]);
+  // The list moves into registers (entry i in lane i % 64 of register i / 64) so that the hot
+  // loop can look slots up with v_readlane instead of an LDS read it would have to wait for.
+  int visr[(WE_MAX_SLOTS + 64) / 64];
+#pragma unroll
+  for (int k = 0; k < (WE_MAX_SLOTS + 64) / 64; ++k) visr[k] = (64 * k + lane < nvis) ? vis[64 * k + lane] : 0;
+  auto vis_at = [&](int i) __attribute__((always_inline)) {
+    const int l = i & 63;
+    switch (i >> 6) {
+      case 0: return __builtin_amdgcn_readlane(visr[0], l);
+      case 1: return __builtin_amdgcn_readlane(visr[1], l);
+      case 2: return __builtin_amdgcn_readlane(visr[2], l);
+      case 3: return __builtin_amdgcn_readlane(visr[3], l);
+      default: return __builtin_amdgcn_readlane(visr[4], l);
+    }
+  };
   const int tps = p.T / BN;  // tiles per slot
   const int nt = nvis * tps;
   const int t_begin = (int)((int64_t)split * nt / p.n_splits);
   const int t_end = (int)((int64_t)(split + 1) * nt / p.n_splits);
   const int ntile = t_end - t_begin;
-  // this group's tiles: t_begin + grp + j*GROUPS, j < n_g; every group runs n_iter iterations
-  const int n_g = ntile > grp ? (ntile - grp + GROUPS - 1) / GROUPS : 0;
-  const int n_iter = (ntile + GROUPS - 1) / GROUPS;
 
   // ---- Q fragments stay in registers, pre-multiplied by scale*log2(e) ----
   const float c2 = p.scale_log2;
   frag_t qf[KS];
-  const int qrow = qtile * BM + wig * 32 + l32;
+  const int qrow = qtile * BM + qb * 32 + l32;
   {
     const uint16_t* qbase = reinterpret_cast<const uint16_t*>(p.q) + b * p.qs_b + h * p.qs_h;
     const int qr = qrow < p.T ? qrow : p.T - 1;
@@ -161,78 +192,68 @@ __global__ void __launch_bounds__(512, 2) attn_ring8_kernel(AttnParams p) {
   const uint64_t vbase = kbase + (uint64_t)((int64_t)p.B * p.Hkv * cap) * ROW_B;
 
   // ---- DMA plumbing ----
-  // Instruction i of this wavefront moves rows [q*RPI, (q+1)*RPI) of a tile, q = wig + i*WPG.
+  // Instruction i of this wavefront moves rows [q*RPI, (q+1)*RPI) of a tile, q = wave + 8*i.
   uint32_t kvoff[NDMA], vvoff[NDMA];
 #pragma unroll
   for (int i = 0; i < NDMA; ++i) {
-    const int row = (wig + i * WPG) * RPI + lane / CPR;
+    const int row = (wave + i * 8) * RPI + lane / CPR;
     const int phys = lane % CPR;
     kvoff[i] = row * ROW_B + ((phys ^ k_swz<DH>(row)) << 4);
     vvoff[i] = row * ROW_B + ((phys ^ v_swz<DH>(row)) << 4);
   }
-  const uint32_t k_ring = lds0 + grp * NST * TILE_B;              // this group's K slots
-  const uint32_t v_ring = lds0 + L::V_OFF + grp * NST * TILE_B;   // this group's V slots
   struct TileWalk {  // position of a load stream in the split's list of visible tiles
     int sidx, sub, left;
   };
-  auto walk_init = [&](int j) __attribute__((always_inline)) {  // group-local tile j (clamped)
+  auto walk_init = [&]() __attribute__((always_inline)) {
     TileWalk w;
-    const int last = n_g > 0 ? n_g - 1 : 0;
-    const int jc = j < last ? j : last;
-    int g = t_begin + grp + jc * GROUPS;
-    if (g >= t_end) g = t_end - 1;  // group without tiles: any valid tile, its result is discarded
-    w.sidx = g / tps;
-    w.sub = g - w.sidx * tps;
-    w.left = last - jc;
+    w.sidx = t_begin / tps;
+    w.sub = t_begin - w.sidx * tps;
+    w.left = ntile - 1;
     return w;
   };
-  auto walk_next = [&](TileWalk& w) __attribute__((always_inline)) {
+  auto walk_next = [&](TileWalk& w) __attribute__((always_inline)) {  // stays on the last tile
     if (w.left > 0) {
       --w.left;
-      w.sub += GROUPS;
-      while (w.sub >= tps) {
-        w.sub -= tps;
+      if (++w.sub == tps) {
+        w.sub = 0;
         ++w.sidx;
       }
     }
   };
   auto tile_base = [&](uint64_t base, const TileWalk& w) __attribute__((always_inline)) {
-    const int slot = __builtin_amdgcn_readfirstlane(vis[w.sidx]);
+    const int slot = vis_at(w.sidx);
     const int64_t row0 = (int64_t)slot * p.T + (int64_t)w.sub * BN;
     return uniform64(base + (uint64_t)row0 * ROW_B);
   };
-  auto dma_k = [&](const TileWalk& w, int slot) __attribute__((always_inline)) {
-    const uint64_t g = tile_base(kbase, w);
+  auto dma_tile = [&](uint64_t base, const uint32_t(&voff)[NDMA], const TileWalk& w, uint32_t lds_tile)
+                      __attribute__((always_inline)) {
+    const uint64_t g = tile_base(base, w);
 #pragma unroll
     for (int i = 0; i < NDMA; ++i)
-      dma16(g, kvoff[i], __builtin_amdgcn_readfirstlane(k_ring + slot * TILE_B + (wig + i * WPG) * 1024));
+      dma16(g, voff[i], __builtin_amdgcn_readfirstlane(lds_tile + (wave + i * 8) * 1024));
+  };
+  auto dma_k = [&](const TileWalk& w, int slot) __attribute__((always_inline)) {
+    dma_tile(kbase, kvoff, w, lds0 + slot * TILE_B);
   };
   auto dma_v = [&](const TileWalk& w, int slot) __attribute__((always_inline)) {
-    const uint64_t g = tile_base(vbase, w);
-#pragma unroll
-    for (int i = 0; i < NDMA; ++i)
-      dma16(g, vvoff[i], __builtin_amdgcn_readfirstlane(v_ring + slot * TILE_B + (wig + i * WPG) * 1024));
+    dma_tile(vbase, vvoff, w, lds0 + L::V_OFF + slot * TILE_B);
   };
 
-  // ---- fragment read addresses (bytes from smem) ----
-  // K row l32 (+32 per key block), logical chunk 2*ks + hh: physical chunk bits [3:1] are
+  // ---- fragment read addresses (byte offsets into smem) ----
+  // K row l32 of a key block, logical chunk 2*ks + hh: physical chunk bits [3:1] are
   // ks ^ (swz >> 1), so the address for step ks is the step-0 address with bits 5.. flipped.
-  uint32_t k_rd[KS];
+  uint32_t k_rd;
   {
     const int x = k_swz<DH>(l32);
-    const uint32_t a0 = grp * NST * TILE_B + l32 * ROW_B + ((((x >> 1) << 1) | (hh ^ (x & 1))) << 4);
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) k_rd[ks] = a0 ^ (ks << 5);
+    k_rd = hb * KB_B + l32 * ROW_B + ((((x >> 1) << 1) | (hh ^ (x & 1))) << 4);
   }
   // V rows 4*hh + r (r = lane bits 3:2) of each 8-row group, logical chunk 4*db + c.
-  uint32_t v_rd[DB];
+  uint32_t v_rd;
   {
     const int r = 4 * hh + ((lane & 15) >> 2);
     const int y = v_swz<DH>(r) >> 2;
     const int c = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-      v_rd[db] = L::V_OFF + grp * NST * TILE_B + r * ROW_B + (((db ^ y) * 4 + c) << 4) + (lane & 1) * 8;
+    v_rd = L::V_OFF + hb * KB_B + r * ROW_B + ((y * 4 + c) << 4) + (lane & 1) * 8;
   }
 
   f32x16_t o[DB];
@@ -243,7 +264,7 @@ __global__ void __launch_bounds__(512, 2) attn_ring8_kernel(AttnParams p) {
   float m_ref = -INFINITY, l_run = 0.f;
 
   const f32x16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  const float kDead = 3.0e4f;  // shift of logits that must not count (tiles past the group's end)
+  const float kDead = 3.0e4f;  // shift of logits that must not count (tiles past the end)
   // K-side fragment of the shift product: contraction index 0 is one for every key
   frag_t ones_frag = __builtin_bit_cast(frag_t, u32x4_t{0u, 0u, 0u, 0u});
   if (hh == 0) ones_frag[0] = (typename M::elem_t)1.0f;
@@ -256,226 +277,272 @@ __global__ void __launch_bounds__(512, 2) attn_ring8_kernel(AttnParams p) {
     if (hh == 0) shift[0] = (typename M::elem_t)(-m_ref);
   };
 
-  // logits of the 64-key tile in K slot `slot`, starting from `init` (a shift product or zero)
-  auto logits = [&](f32x16_t(&s)[2], int slot, bool shifted, const frag_t& sh) __attribute__((always_inline)) {
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-      s[kb] = shifted ? M::mma(ones_frag, sh, zero16) : zero16;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const frag_t a = *reinterpret_cast<const frag_t*>(smem + k_rd[ks] + slot * TILE_B + kb * 32 * ROW_B);
-        s[kb] = M::mma(a, qf[ks], s[kb]);
-      }
-    }
-  };
-  // O^T += V^T P^T for the tile in V slot `slot`
-  auto accumulate = [&](const frag_t(&pf)[4], int slot) __attribute__((always_inline)) {
-#pragma unroll
-    for (int m = 0; m < 4; ++m) {
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        const unsigned char* va = smem + v_rd[db] + slot * TILE_B + 16 * m * ROW_B;
-        const s16x4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(va));
-        const s16x4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(va + 8 * ROW_B));
-        typedef short s16x8_t __attribute__((ext_vector_type(8)));
-        const s16x8_t a8 = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
-        o[db] = M::mma(__builtin_bit_cast(frag_t, a8), pf[m], o[db]);
-      }
-    }
-  };
-  // probabilities of one tile from its shifted logits: p = 2^(s - sub), packed to the element
-  // type; returns this half-wave's share of the row sum (of the rounded values)
-  auto probabilities = [&](frag_t(&pf)[4], const f32x16_t(&s)[2], float sub) __attribute__((always_inline)) {
+  // probabilities of one 32-key block from its shifted logits: p = 2^(s - sub), packed to the
+  // element type; returns this half-wave's share of the row sum (of the rounded values)
+  auto probabilities = [&](frag_t(&pf)[2], const f32x16_t& s, float sub) __attribute__((always_inline)) {
     float rs = 0.f;
 #pragma unroll
-    for (int m = 0; m < 4; ++m) {
-      const f32x16_t& sv = s[m >> 1];
-      const int r0 = 8 * (m & 1);
+    for (int m = 0; m < 2; ++m) {
       float e[8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) e[j] = __builtin_amdgcn_exp2f(sv[r0 + j] - sub);
+      for (int j = 0; j < 8; ++j) e[j] = __builtin_amdgcn_exp2f(s[8 * m + j] - sub);
       pf[m] = M::pack8(e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7]);
 #pragma unroll
       for (int j = 0; j < 4; ++j) rs = M::add_pair(rs, pf[m], j);
     }
     return rs;
   };
-  auto tile_max = [&](const f32x16_t(&s)[2]) __attribute__((always_inline)) {
-    float mx = s[0][0];
+  auto block_max = [&](const f32x16_t& s) __attribute__((always_inline)) {
+    float mx = s[0];
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kb][i]);
+    for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s[i]);
     float lo, up;
     half_wave_pair(mx, lo, up);
     return fmaxf(lo, up);
   };
 
-  if (ntile > 0) {
-    frag_t p_prev[4];
-    f32x16_t s_cur[2];
-    {
-      // zero the V slot that stands in for "tile -1" and P, so the first product adds zeros
-      const u32x4_t z = {0u, 0u, 0u, 0u};
-      unsigned char* vz = smem + L::V_OFF + (grp * NST + NST - 1) * TILE_B;
-      for (int i = wig * 64 + lane; i < TILE_B / 16; i += WPG * 64) *reinterpret_cast<u32x4_t*>(vz + i * 16) = z;
-#pragma unroll
-      for (int m = 0; m < 4; ++m) p_prev[m] = __builtin_bit_cast(frag_t, z);
-    }
-    // Prologue issue order mirrors the loop's (K(j+NST), V(j+NST-2) in iteration j).
-    TileWalk kw = walk_init(0), vw = walk_init(0);
-    if (NST == 4) {
-      dma_k(kw, 0); walk_next(kw);
-      dma_k(kw, 1); walk_next(kw);
-      dma_k(kw, 2); walk_next(kw);
-      dma_v(vw, 0); walk_next(vw);
-      dma_k(kw, 3); walk_next(kw);
-      dma_v(vw, 1); walk_next(vw);
-      dma_wait<5 * NDMA>();
+  // The pipeline runs on 32-key blocks.  One step computes, for this wavefront,
+  //   matrix cores: the shifted logits of the block read at K offset KOFF (-> s_next) and the
+  //                 product of the previous block's probabilities with the V block at VOFF;
+  //   VALU:         the probabilities of the current block (s_cur -> p_cur).
+  // LDS reads are issued in consumption order - K fragments 0..KS-1, then the NV V^T fragments
+  // (two transposing reads each) - running up to 15 reads ahead of the MFMAs.
+  bool pending = false;   // an accumulator rescale decided in the previous step is due
+  float alpha = 1.f;
+  frag_t p_prev[2];
+  f32x16_t s_cur;
+  // Fragment registers live across steps: every step starts with its first PRE reads (all K
+  // fragments and the first V^T fragment) already in flight, issued during the previous step.
+  constexpr int PRE = KS + 2;
+  u32x4_t kf[KS];
+  u32x2_t v0[NV], v1[NV];
+  auto read_k = [&](auto koff_c, int ks) __attribute__((always_inline)) {
+    kf[ks] = lds_read128<decltype(koff_c)::value>(smem, k_rd ^ (ks << 5));
+  };
+  auto read_v = [&](auto voff_c, int i) __attribute__((always_inline)) {  // fragment i = (m, db) = (i / DB, i % DB)
+    constexpr int VOFF = decltype(voff_c)::value;
+    const uint32_t a = v_rd ^ ((i % DB) << 6);
+    if (i / DB == 0) {
+      v0[i] = lds_read_tr<VOFF>(smem, a);
+      v1[i] = lds_read_tr<VOFF + 8 * ROW_B>(smem, a);
     } else {
-      dma_k(kw, 0); walk_next(kw);
-      dma_k(kw, 1); walk_next(kw);
-      dma_wait<NDMA>();
+      v0[i] = lds_read_tr<VOFF + 16 * ROW_B>(smem, a);
+      v1[i] = lds_read_tr<VOFF + 24 * ROW_B>(smem, a);
     }
-    __syncthreads();  // K(0) and the zeroed V slot are in LDS
-    // first tile: plain logits, reference = its row max, shifted by hand
-    logits(s_cur, 0, false, shift);
-    if (n_g > 0) {
-      m_ref = M::round_up(tile_max(s_cur));
-      set_shift();
+  };
+  auto prefetch = [&](auto koff_c, auto voff_c) __attribute__((always_inline)) {
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) s_cur[kb][i] -= m_ref;
-    } else {  // this group has no tile of its own: everything it computes is weighted 2^-kDead
-      m_ref = 0.f;
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) s_cur[kb][i] = -kDead;
-    }
-    if (NST == 4) dma_wait<4 * NDMA>(); else dma_wait<0>();
-    __syncthreads();  // K(1) landed; K slot 0 may be overwritten
-
-    // A raise decided in iteration j rescales the accumulators after the product of tile j-1
-    // and before that of tile j, i.e. at the top of iteration j+1; with the branch there the
-    // rest of the body stays one basic block for the scheduler to interleave.
-    bool pending = false;
-    float alpha = 1.f;
-    auto rescale = [&]() __attribute__((always_inline)) {
+    for (int ks = 0; ks < KS; ++ks) read_k(koff_c, ks);
+    read_v(voff_c, 0);
+  };
+  auto step = [&](auto koff_c, auto voff_c, auto nkoff_c, auto nvoff_c, bool live, auto&& mid) __attribute__((always_inline)) {
+    if (pending) {
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
         for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+    }
+    pending = false;
+
+    // reads issued since this step's read 0 / next own V fragment / next-step read pairs issued
+    int issued = PRE, vnext = 1, npair = 0;
+    constexpr int NPAIR = PRE / 2;            // the next step's first reads go out two at a time
+    constexpr int I0 = NV - 1 - NPAIR;        // ... after the product MFMAs I0, I0+1, ...
+    auto next_pair = [&]() __attribute__((always_inline)) {
+      if (2 * npair < KS) {
+        read_k(nkoff_c, 2 * npair);
+        read_k(nkoff_c, 2 * npair + 1);
+      } else {
+        read_v(nvoff_c, 0);
+      }
+      ++npair;
+      issued += 2;
     };
 
-    // one iteration with compile-time ring positions (JM = j mod NST)
+    // From here to the end of the product the issue order is pinned statement by statement
+    // (sched_barrier): MFMA, the reads that refill the queue, a slice of the VALU work.
+    __builtin_amdgcn_sched_barrier(0);
+    f32x16_t s_next = M::mma(ones_frag, live ? shift : dead, zero16);
+    frag_t p_cur[2];
+    float e[16];
+    float rs = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      s_next = M::mma(__builtin_bit_cast(frag_t, kf[ks]), qf[ks], s_next);
+      // keep the read queue full without exceeding the 15 reads the counter can track
+      if (vnext < NV && ks <= 12 - KS) {
+        read_v(voff_c, vnext);
+        ++vnext;
+        issued += 2;
+      }
+      // VALU slice: 16 / KS exponentials of the current block
+#pragma unroll
+      for (int t = 0; t < 16 / KS; ++t)
+        e[ks * (16 / KS) + t] = __builtin_amdgcn_exp2f(s_cur[ks * (16 / KS) + t]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    mid();  // the tile DMAs of this iteration go out here, under the MFMAs already queued
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      if (vnext < NV) {  // reads 0..KS+2i-1 have completed: room for one more fragment
+        read_v(voff_c, vnext);
+        ++vnext;
+        issued += 2;
+      }
+      typedef unsigned int u32x4v __attribute__((ext_vector_type(4)));
+      const u32x4v a4 = __builtin_shufflevector(v0[i], v1[i], 0, 1, 2, 3);
+      o[i % DB] = M::mma(__builtin_bit_cast(frag_t, a4), p_prev[i / DB], o[i % DB]);
+      if (i >= I0 && npair < NPAIR) next_pair();
+      // VALU slices: pack the two 16-key halves, then their row sums
+      if (i == 0) p_cur[0] = M::pack8(e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7]);
+      if (i == 1) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) rs = M::add_pair(rs, p_cur[0], t);
+      }
+      if (i == 2) p_cur[1] = M::pack8(e[8], e[9], e[10], e[11], e[12], e[13], e[14], e[15]);
+      if (i == 3) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) rs = M::add_pair(rs, p_cur[1], t);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+
+    if (__ballot(!(rs <= 256.f)) != 0ull) {
+      // Rare: some probability of this block may exceed 2^8.  Raise the reference of the rows
+      // that need it, redo the block's probabilities exactly, and re-base the logits of the next
+      // block, which were produced with the old reference.
+      const float mx = block_max(s_cur);
+      const float m_new = mx > 0.f ? M::round_up(m_ref + mx) : m_ref;
+      const float delta = m_new - m_ref;
+      alpha = __builtin_amdgcn_exp2f(-delta);
+      rs = probabilities(p_cur, s_cur, delta);
+      l_run *= alpha;
+      m_ref = m_new;
+      set_shift();
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s_next[i] -= delta;
+      pending = true;
+    }
+    l_run += rs;
+    p_prev[0] = p_cur[0];
+    p_prev[1] = p_cur[1];
+    s_cur = s_next;
+  };
+
+  if (ntile > 0) {
+    {
+      // zero V slot 3, which stands in for "tile -1", and P, so the first product adds zeros
+      const u32x4_t z = {0u, 0u, 0u, 0u};
+      unsigned char* vz = smem + L::V_OFF + 3 * TILE_B;
+      for (int i = tid; i < TILE_B / 16; i += 512) *reinterpret_cast<u32x4_t*>(vz + i * 16) = z;
+      p_prev[0] = __builtin_bit_cast(frag_t, z);
+      p_prev[1] = __builtin_bit_cast(frag_t, z);
+    }
+    // Iteration j issues K(j+KA) and V(j+2) (KA = 3, or 4 when every wavefront handles one key
+    // block per tile and prefetches its next fragments across the barrier); the prologue issues
+    // what the iterations before 0 would have.
+    constexpr int KA = KSPLIT == 1 ? 3 : 4;
+    TileWalk kw = walk_init(), vw = walk_init();
+    dma_k(kw, 0); walk_next(kw);
+    dma_k(kw, 1); walk_next(kw);
+    if (KSPLIT == 2) { dma_k(kw, 2); walk_next(kw); }
+    dma_v(vw, 0); walk_next(vw);
+    dma_k(kw, KA - 1); walk_next(kw);
+    dma_v(vw, 1); walk_next(vw);
+    dma_wait<(KA + 1) * NDMA>();
+    __syncthreads();  // K(0) and the zeroed V slot are in LDS
+    // first block: plain logits, reference = its row max, shifted by hand
+    {
+      s_cur = zero16;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const frag_t a = *reinterpret_cast<const frag_t*>(smem + (k_rd ^ (ks << 5)));
+        s_cur = M::mma(a, qf[ks], s_cur);
+      }
+      m_ref = M::round_up(block_max(s_cur));
+      set_shift();
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s_cur[i] -= m_ref;
+    }
+    dma_wait<2 * NDMA>();
+    __syncthreads();  // everything but the last K and V tile issued so far has landed
+    // first reads of the first step
+    if (KSPLIT == 1) prefetch(IntC<KB_B>(), IntC<3 * TILE_B + KB_B>());
+    else prefetch(IntC<TILE_B>(), IntC<3 * TILE_B>());
+
+    // one tile iteration with compile-time ring positions (JM = j mod 4)
     auto iteration = [&](int j, auto jm_c) __attribute__((always_inline)) {
       constexpr int JM = decltype(jm_c)::value;
-      if (pending) rescale();
-      pending = false;
-      dma_k(kw, JM);                          // K(j+NST)
-      walk_next(kw);
-      dma_v(vw, (JM + NST - 2) % NST);        // V(j+NST-2)
-      walk_next(vw);
-
-      // matrix cores: shifted logits of tile j+1 (weighted out if past this group's end)
-      f32x16_t s_next[2];
-      logits(s_next, (JM + 1) % NST, true, (j + 1 < n_g) ? shift : dead);
-
-      // VALU: probabilities of tile j
-      frag_t p_cur[4];
-      float rs = probabilities(p_cur, s_cur, 0.f);
-
-      // matrix cores: O += P(j-1) V(j-1)
-      accumulate(p_prev, (JM + NST - 1) % NST);
-
-      // Issue order for the block above: keep several LDS fragment reads in flight ahead of the
-      // MFMA that consumes them and spread the vector work between the MFMAs.
-      __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
-#pragma unroll
-      for (int i = 0; i < 6; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+      auto issue_dma = [&]() __attribute__((always_inline)) {
+        dma_k(kw, (JM + KA) % NST);  // K(j+KA)
+        walk_next(kw);
+        dma_v(vw, (JM + 2) % NST);   // V(j+2)
+        walk_next(vw);
+      };
+      auto nothing = [&]() __attribute__((always_inline)) {};
+      if (KSPLIT == 1) {
+        // block (j, 0) -> probabilities; logits of (j, 1); product of (j-1, 1)
+        step(IntC<JM * TILE_B + KB_B>(), IntC<((JM + 3) % NST) * TILE_B + KB_B>(),
+             IntC<((JM + 1) % NST) * TILE_B>(), IntC<JM * TILE_B>(), true, issue_dma);
+        // block (j, 1) -> probabilities; logits of (j+1, 0); product of (j, 0)
+        step(IntC<((JM + 1) % NST) * TILE_B>(), IntC<JM * TILE_B>(),
+             IntC<((JM + 1) % NST) * TILE_B + KB_B>(), IntC<JM * TILE_B + KB_B>(), j + 1 < ntile, nothing);
+      } else {
+        // block (j, hb) -> probabilities; logits of (j+1, hb); product of (j-1, hb)
+        step(IntC<((JM + 1) % NST) * TILE_B>(), IntC<((JM + 3) % NST) * TILE_B>(),
+             IntC<((JM + 2) % NST) * TILE_B>(), IntC<JM * TILE_B>(), j + 1 < ntile, issue_dma);
       }
-#pragma unroll
-      for (int i = 6; i < 2 * KS + 2 + 4 * DB; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
-      }
-
-      if (__ballot(!(rs <= 256.f)) != 0ull) {
-        // Rare: some probability of this tile may exceed 2^8.  Raise the reference of the rows
-        // that need it, redo the tile's probabilities exactly, and re-base the logits of the
-        // next tile, which were produced with the old reference.
-        const float mx = tile_max(s_cur);
-        const float m_new = mx > 0.f ? M::round_up(m_ref + mx) : m_ref;
-        const float delta = m_new - m_ref;
-        alpha = __builtin_amdgcn_exp2f(-delta);
-        rs = probabilities(p_cur, s_cur, delta);
-        l_run *= alpha;
-        m_ref = m_new;
-        set_shift();
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) s_next[kb][i] -= delta;
-        pending = true;
-      }
-      l_run += rs;
-#pragma unroll
-      for (int m = 0; m < 4; ++m) p_prev[m] = p_cur[m];
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb) s_cur[kb] = s_next[kb];
-      dma_wait<(NST - 2) * 2 * NDMA>();  // K(j+2) and V(j) have landed (this wavefront's part)
+      dma_wait<2 * NDMA>();  // all but this iteration's two tiles have landed (this wavefront's part)
       __syncthreads();
     };
 
     int j = 0;
-    if (NST == 4) {
-      for (; j + 4 <= n_iter; j += 4) {
-        iteration(j, IntC<0>());
-        iteration(j + 1, IntC<1>());
-        iteration(j + 2, IntC<2>());
-        iteration(j + 3, IntC<3>());
-      }
-      if (j < n_iter) { iteration(j, IntC<0>()); ++j; }
-      if (j < n_iter) { iteration(j, IntC<1>()); ++j; }
-      if (j < n_iter) { iteration(j, IntC<2>()); ++j; }
-    } else {
-      for (; j + 2 <= n_iter; j += 2) {
-        iteration(j, IntC<0>());
-        iteration(j + 1, IntC<1>());
-      }
-      if (j < n_iter) { iteration(j, IntC<0>()); ++j; }
+    for (; j + 4 <= ntile; j += 4) {
+      iteration(j, IntC<0>());
+      iteration(j + 1, IntC<1>());
+      iteration(j + 2, IntC<2>());
+      iteration(j + 3, IntC<3>());
     }
-    if (pending) rescale();
-    // product of the last tile: V(n_iter-1) sits in slot (n_iter-1) mod NST
+    if (j < ntile) { iteration(j, IntC<0>()); ++j; }
+    if (j < ntile) { iteration(j, IntC<1>()); ++j; }
+    if (j < ntile) { iteration(j, IntC<2>()); ++j; }
+
+    // product of the last block: (ntile-1, 1) for full-tile wavefronts, (ntile-1, hb) otherwise
+    if (pending) {
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+    }
     {
-      const int last = (n_iter - 1) % NST;
-      if (last == 0) accumulate(p_prev, 0);
-      else if (last == 1) accumulate(p_prev, 1);
-      else if (NST == 4 && last == 2) accumulate(p_prev, 2);
-      else accumulate(p_prev, NST - 1);
+      const int last = (ntile - 1) % NST;
+      const unsigned char* vt = smem + v_rd + last * TILE_B + (KSPLIT == 1 ? KB_B : 0);
+#pragma unroll
+      for (int m = 0; m < 2; ++m) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const unsigned char* va = smem + ((uint32_t)(vt - smem) ^ (db << 6)) + 16 * m * ROW_B;
+          const s16x4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(va));
+          const s16x4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(va + 8 * ROW_B));
+          typedef short s16x8_t __attribute__((ext_vector_type(8)));
+          const s16x8_t a8 = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
+          o[db] = M::mma(__builtin_bit_cast(frag_t, a8), p_prev[m], o[db]);
+        }
+      }
     }
     dma_wait<0>();  // no DMA may still be writing LDS when the rings are reused or the CU is freed
-  }
-  if (n_g == 0) {
-    m_ref = -INFINITY;
-    l_run = 0.f;
   }
 
   float lo, up;
   half_wave_pair(l_run, lo, up);
   float l_tot = lo + up;
 
-  if (GROUPS == 2) {
-    // ---- merge the two groups' (m, l, O) through LDS; group 0 keeps the result ----
+  if (KSPLIT == 2) {
+    // ---- the two wavefronts of a query block merge their (m, l, O) through LDS ----
     __syncthreads();  // every wavefront is done with the rings
-    float* mb = reinterpret_cast<float*>(smem) + (wig * (DB * 16 + 2)) * 64 + lane;
-    if (grp == 1) {
+    float* mb = reinterpret_cast<float*>(smem) + (qb * (DB * 16 + 2)) * 64 + lane;
+    if (hb == 1) {
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -484,7 +551,7 @@ __global__ void __launch_bounds__(512, 2) attn_ring8_kernel(AttnParams p) {
       mb[(DB * 16 + 1) * 64] = l_tot;
     }
     __syncthreads();
-    if (grp == 1) return;
+    if (hb == 1) return;
     const float m1 = mb[(DB * 16) * 64], l1 = mb[(DB * 16 + 1) * 64];
     const float mm = fmaxf(m_ref, m1);
     if (mm > -INFINITY) {
@@ -537,19 +604,19 @@ __global__ void __launch_bounds__(512, 2) attn_ring8_kernel(AttnParams p) {
   }
 }
 
-template <typename M, int DH, int GROUPS>
+template <typename M, int DH, int KSPLIT>
 static hipError_t launch_ring8_t(const AttnParams& p, hipStream_t stream) {
   static bool configured = false;
   const int lds = Ring8Lds<DH>::kBytes;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_ring8_kernel<M, DH, GROUPS>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_ring8_kernel<M, DH, KSPLIT>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
     configured = true;
   }
   const int rounds = (p.unit_splits + 7) / 8;
   const unsigned grid = (unsigned)(rounds * 8 * p.members);
-  hipLaunchKernelGGL((attn_ring8_kernel<M, DH, GROUPS>), dim3(grid), dim3(512), lds, stream, p);
+  hipLaunchKernelGGL((attn_ring8_kernel<M, DH, KSPLIT>), dim3(grid), dim3(512), lds, stream, p);
   return hipGetLastError();
 }
 

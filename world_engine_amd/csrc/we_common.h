@@ -11,6 +11,7 @@ typedef short s16x4_t __attribute__((ext_vector_type(4)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
 
 // Floor division / modulo on int64, the semantics of `//` and `%` on torch int64 tensors
 // (src/model/kv_cache.py:129-130,140).
