@@ -62,6 +62,7 @@ def main():
     ap.add_argument("--eager", action="store_true", help="launch from Python per call instead of a HIP graph")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--attn-iters", type=int, default=200, help="attention-only launches for the roofline timing")
+    ap.add_argument("--batch", type=int, default=0, help="override the configuration's batch size (experiments)")
     args = ap.parse_args()
 
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -75,7 +76,10 @@ def main():
     import world_engine_amd as wea
     from world_engine_amd import ops
 
-    c = CONFIGS[args.config]
+    c = dict(CONFIGS[args.config])
+    if args.batch:
+        c["B"] = args.batch
+        c["name"] += f" [batch overridden to {args.batch}]"
     B, H, Hkv, Dh, T, n, layers = c["B"], c["H"], c["Hkv"], c["Dh"], c["T"], c["slots"], c["layers"]
     L = n * T
     W = int(math.isqrt(T))
@@ -112,7 +116,7 @@ def main():
     t_pos_all = torch.arange(frames_total, dtype=torch.long)[:, None, None].expand(frames_total, B, T).contiguous().to(dev)
 
     n_splits = args.n_splits or ops.attn_auto_splits(B, H, Hkv, T, Dh, L)
-    ws = torch.empty(max(ops.attn_workspace_bytes(B, H, T, Dh, n_splits), 16), dtype=torch.uint8, device=dev)
+    ws = torch.empty(max(ops.attn_workspace_bytes(B, H, Hkv, T, Dh, L, args.n_splits, args.q_tile), 16), dtype=torch.uint8, device=dev)
     out = torch.empty((B, T, H, Dh), dtype=dtype, device=dev).transpose(1, 2)
 
     def one_step(step_idx):
@@ -125,7 +129,7 @@ def main():
             q, k, v = inputs[(step_idx + li) % n_in]
             q_rot = ops.rope_kv_store(q, k, v, pos, rope.cos, rope.sin, rope.height, rope.width,
                                       layer.kv, layer.written, layer.L, 1, frozen)
-            ops.attn_ring(q_rot, layer.kv, layer.written, pos["t_pos"], layer.L, 1, n_splits=n_splits,
+            ops.attn_ring(q_rot, layer.kv, layer.written, pos["t_pos"], layer.L, 1, n_splits=args.n_splits,
                           q_tile=args.q_tile, out=out, workspace=ws)
 
     # ---- fill the ring (untimed, not counted), then W warm-up steps ----
@@ -169,7 +173,7 @@ def main():
     iters = args.attn_iters
 
     def attn_only():
-        ops.attn_ring(q_rot, layer0.kv, layer0.written, pos["t_pos"], layer0.L, 1, n_splits=n_splits,
+        ops.attn_ring(q_rot, layer0.kv, layer0.written, pos["t_pos"], layer0.L, 1, n_splits=args.n_splits,
                       q_tile=args.q_tile, out=out, workspace=ws)
 
     for _ in range(5):

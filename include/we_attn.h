@@ -102,14 +102,18 @@ int we_rope_apply(const void* x, const int64_t x_strides[3], void* x_out,
                   int32_t B, int32_t H, int32_t T, int32_t Dh, int32_t dtype, void* stream);
 
 /*
- * Number of context splits we_attn_ring_fwd picks when called with n_splits = 0.
+ * Number of context parts we_attn_ring_fwd cuts split units into when called with n_splits = 0
+ * (1 = nothing is split).  Sizing helper without a counterpart in the reference.
  */
 int32_t we_attn_auto_splits(int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L);
 
 /*
- * Bytes of workspace we_attn_ring_fwd needs for a given split count (0 when n_splits <= 1).
+ * Bytes of split-context workspace we_attn_ring_fwd needs for these sizes and the given n_splits /
+ * q_tile arguments (0 when nothing is split).  Sizing helper without a counterpart in the
+ * reference.
  */
-size_t we_attn_workspace_bytes(int32_t B, int32_t H, int32_t T, int32_t Dh, int32_t n_splits);
+size_t we_attn_workspace_bytes(int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L,
+                               int32_t n_splits, int32_t q_tile);
 
 /*
  * Frame-block-causal attention of one frame's queries over the ring buffer.
@@ -125,11 +129,16 @@ size_t we_attn_workspace_bytes(int32_t B, int32_t H, int32_t T, int32_t Dh, int3
  *   q    [B, H, T, Dh]   element strides q_strides = {batch, head, token}; Dh contiguous.
  *   kv, written, t_pos   as in we_rope_kv_store, after that call for the same frame.
  *   out  [B, H, T, Dh]   element strides out_strides = {batch, head, token}; Dh contiguous.
- *   workspace            device scratch of at least we_attn_workspace_bytes(..., n_splits)
- *                        bytes when the effective split count is > 1; may be NULL otherwise.
- *   n_splits             0 = choose automatically; 1 = single pass; 2..64 = split the visible
- *                        context into that many parts and combine them in a second kernel.
- *   q_tile               queries per workgroup: 0 = choose automatically, or 128 / 256.
+ *   workspace            device scratch of at least we_attn_workspace_bytes(...) bytes for the
+ *                        same sizes, n_splits and q_tile; may be NULL when that is 0.
+ *   n_splits             0 = choose automatically (small grids: every (batch, kv head) unit is
+ *                        split so that all CUs have work; grids that leave a partial last round
+ *                        of workgroups: only that round's units are split); 1 = single pass;
+ *                        2..64 = split the visible context of every unit into that many parts.
+ *                        Split parts are combined by a second kernel.
+ *   q_tile               kernel shape: 0 = choose automatically; 129 / 257 = 8-wavefront
+ *                        LDS-DMA kernel with 128 / 256 queries per workgroup; 128 / 256 =
+ *                        4-wavefront register-staged kernel with 128 / 256 queries.
  *   scale                softmax scale (> 0); the reference uses 1/sqrt(Dh).
  *
  * Requirements: dtype bf16 or f16; Dh in {64, 128}; T % 64 == 0; L/T <= WE_MAX_SLOTS;

@@ -144,6 +144,15 @@ def test_attention_dtypes_head_dims_and_ragged_tiles(gpu_device, dtype, Dh, T):
         _run_and_check(p, 5, **kw)
 
 
+def test_attention_partial_round_tail_split(gpu_device):
+    """320 workgroups = one full round of 256 CUs plus a quarter round: the library splits the
+    context of the last 32 heads only (mixed direct-output and workspace rows in one call)."""
+    assert ops.attn_auto_splits(1, 160, 160, 256, 64, 512) == 2
+    assert ops.attn_workspace_bytes(1, 160, 160, 256, 64, 512) == 2 * 32 * 256 * (64 + 2) * 4
+    p = Pair(gpu_device, torch.bfloat16, B=1, H=160, Hkv=160, T=256, Dh=64, n_slots=2, cfg_id=27)
+    _run_and_check(p, 4)
+
+
 @pytest.mark.parametrize("d", [2, 4])
 def test_attention_with_pinned_dilation(gpu_device, d):
     p = Pair(gpu_device, torch.bfloat16, B=1, H=2, Hkv=2, T=64, Dh=128, n_slots=4 * d, d=d, cfg_id=23)
@@ -279,7 +288,7 @@ def test_hip_graph_replay_matches_eager(gpu_device):
     layer = p.hip.layers[0]
     out_s = torch.empty(1, 4, 128, 128, dtype=torch.bfloat16, device=dev)
     n_splits = 2
-    ws = torch.empty(ops.attn_workspace_bytes(1, 4, 128, 128, n_splits), dtype=torch.uint8, device=dev)
+    ws = torch.empty(ops.attn_workspace_bytes(1, 4, 4, 128, 128, layer.L, n_splits), dtype=torch.uint8, device=dev)
 
     def step():
         q_rot = ops.rope_kv_store(qs, ks, vs, pos_s, p.rope.cos, p.rope.sin, p.Hgrid, p.W, layer.kv,

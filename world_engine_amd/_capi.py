@@ -41,7 +41,7 @@ SIGNATURES = {
         c_int32, c_void_p,                         # dtype, stream
     ]),
     "we_attn_auto_splits": (c_int32, [c_int32, c_int32, c_int32, c_int32, c_int32, c_int64]),
-    "we_attn_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32, c_int32]),
+    "we_attn_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32, c_int32, c_int64, c_int32, c_int32]),
     "we_attn_ring_fwd": (c_int32, [
         c_void_p, _I64x3,                          # q, q_strides
         c_void_p, c_void_p, c_void_p,              # kv, written, t_pos

@@ -61,7 +61,14 @@ __global__ void __launch_bounds__(256, NQB == 1 ? 2 : 1) attn_ring_kernel(AttnPa
   const int round = jj / p.members, member = jj - round * p.members;
   const int us = round * 8 + xcd;
   if (us >= p.unit_splits) return;
-  const int unit = us / p.n_splits, split = us - unit * p.n_splits;
+  // leading units run unsplit; the rest are cut into n_splits context parts each
+  int unit, split, nsp;
+  if (us < p.units_whole) {
+    unit = us; split = 0; nsp = 1;
+  } else {
+    const int r = us - p.units_whole;
+    unit = p.units_whole + r / p.n_splits; split = r % p.n_splits; nsp = p.n_splits;
+  }
   const int b = unit / p.Hkv, hkv = unit - b * p.Hkv;
   const int hq_in = member / p.q_tiles, qtile = member - hq_in * p.q_tiles;
   const int h = hkv * (p.H / p.Hkv) + hq_in;
@@ -87,8 +94,8 @@ __global__ void __launch_bounds__(256, NQB == 1 ? 2 : 1) attn_ring_kernel(AttnPa
   const int nvis = vis[WE_MAX_SLOTS + 1];
   const int tps = p.T / BN;  // tiles per slot
   const int nt = nvis * tps;
-  const int t_begin = (int)((int64_t)split * nt / p.n_splits);
-  const int t_end = (int)((int64_t)(split + 1) * nt / p.n_splits);
+  const int t_begin = (int)((int64_t)split * nt / nsp);
+  const int t_end = (int)((int64_t)(split + 1) * nt / nsp);
   const int ntile = t_end - t_begin;
 
   // ---- Q fragments stay in registers for the whole kernel, pre-multiplied by scale*log2(e) so
@@ -379,18 +386,18 @@ __global__ void __launch_bounds__(256, NQB == 1 ? 2 : 1) attn_ring_kernel(AttnPa
   for (int qb = 0; qb < NQB; ++qb) m_run[qb] = m_ref[qb];
 
   // ---- epilogue ----
-  const int64_t rows = (int64_t)p.B * p.H * p.T;
+  const int64_t rows = (int64_t)p.B * p.H * p.T - p.ws_row0;  // rows in the workspace
 #pragma unroll
   for (int qb = 0; qb < NQB; ++qb) {
     float lo, up;
     half_wave_pair(l_run[qb], lo, up);
     const float l_tot = lo + up;
     const bool valid = qrow[qb] < p.T;
-    const float inv = (p.n_splits == 1) ? 1.f / l_tot : 1.f;
+    const float inv = (nsp == 1) ? 1.f / l_tot : 1.f;
     const int64_t row = ((int64_t)b * p.H + h) * p.T + qrow[qb];
-    if (p.n_splits > 1 && valid && hh == 0) {
+    if (nsp > 1 && valid && hh == 0) {
       float2 ml = make_float2(m_run[qb], l_tot);
-      *reinterpret_cast<float2*>(p.ws_ml + ((int64_t)split * rows + row) * 2) = ml;
+      *reinterpret_cast<float2*>(p.ws_ml + ((int64_t)split * rows + (row - p.ws_row0)) * 2) = ml;
     }
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
@@ -409,12 +416,12 @@ __global__ void __launch_bounds__(256, NQB == 1 ? 2 : 1) attn_ring_kernel(AttnPa
         }
         const int d0 = 32 * db + 8 * (c + hh);
         if (valid) {
-          if (p.n_splits == 1) {
+          if (nsp == 1) {
             uint16_t* dst = reinterpret_cast<uint16_t*>(p.out) + b * p.os_b + h * p.os_h +
                             (int64_t)qrow[qb] * p.os_t + d0;
             *reinterpret_cast<frag_t*>(dst) = M::pack8(f[0], f[1], f[2], f[3], f[4], f[5], f[6], f[7]);
           } else {
-            float* dst = p.ws_o + ((int64_t)split * rows + row) * DH + d0;
+            float* dst = p.ws_o + ((int64_t)split * rows + (row - p.ws_row0)) * DH + d0;
             *reinterpret_cast<float4*>(dst) = make_float4(f[0], f[1], f[2], f[3]);
             *reinterpret_cast<float4*>(dst + 4) = make_float4(f[4], f[5], f[6], f[7]);
           }
@@ -428,10 +435,10 @@ __global__ void __launch_bounds__(256, NQB == 1 ? 2 : 1) attn_ring_kernel(AttnPa
 // w_s = 2^(m_s - max_s m_s).  One thread per (query row, 4 head-dim columns).
 template <typename M, int DH>
 __global__ void __launch_bounds__(256) attn_combine_kernel(AttnParams p) {
-  const int64_t rows = (int64_t)p.B * p.H * p.T;
+  const int64_t rows = (int64_t)p.B * p.H * p.T - p.ws_row0;  // rows that were split
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= rows * (DH / 4)) return;
-  const int64_t row = idx / (DH / 4);
+  const int64_t row = idx / (DH / 4);  // workspace row; query row = row + ws_row0
   const int dg = (int)(idx % (DH / 4));
   float mmax = -INFINITY;
   for (int s = 0; s < p.n_splits; ++s) mmax = fmaxf(mmax, p.ws_ml[((int64_t)s * rows + row) * 2]);
@@ -448,19 +455,15 @@ __global__ void __launch_bounds__(256) attn_combine_kernel(AttnParams p) {
     acc.w += w * ov.w;
   }
   const float inv = 1.f / den;
-  const int t = (int)(row % p.T);
-  const int64_t bh = row / p.T;
+  const int64_t qrow = row + p.ws_row0;
+  const int t = (int)(qrow % p.T);
+  const int64_t bh = qrow / p.T;
   const int h = (int)(bh % p.H);
   const int b = (int)(bh / p.H);
   uint16_t* dst = reinterpret_cast<uint16_t*>(p.out) + b * p.os_b + h * p.os_h + (int64_t)t * p.os_t + dg * 4;
   typename M::frag_t pk = M::pack8(acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv, 0.f, 0.f, 0.f, 0.f);
   const uint4 bits = __builtin_bit_cast(uint4, pk);
   *reinterpret_cast<uint2*>(dst) = make_uint2(bits.x, bits.y);
-}
-
-int attn_block_m(int Dh, int variant) {
-  (void)Dh;
-  return variant == 2 ? 256 : 128;
 }
 
 template <typename M, int DH, int NQB>
@@ -492,7 +495,7 @@ hipError_t launch_attn_ring(const AttnParams& p, int Dh, int dtype, int variant,
 }
 
 hipError_t launch_attn_combine(const AttnParams& p, int Dh, int dtype, hipStream_t stream) {
-  const int64_t total = (int64_t)p.B * p.H * p.T * (Dh / 4);
+  const int64_t total = ((int64_t)p.B * p.H * p.T - p.ws_row0) * (Dh / 4);
   const unsigned grid = (unsigned)((total + 255) / 256);
   if (dtype == WE_DTYPE_BF16) {
     if (Dh == 128) hipLaunchKernelGGL((attn_combine_kernel<Bf16Mma, 128>), dim3(grid), dim3(256), 0, stream, p);

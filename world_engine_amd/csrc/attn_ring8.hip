@@ -126,7 +126,14 @@ __global__ void __launch_bounds__(512, 2) attn_ring8_kernel(AttnParams p) {
   const int round = jj / p.members, member = jj - round * p.members;
   const int us = round * 8 + xcd;
   if (us >= p.unit_splits) return;
-  const int unit = us / p.n_splits, split = us - unit * p.n_splits;
+  // leading units run unsplit; the rest are cut into n_splits context parts each
+  int unit, split, nsp;
+  if (us < p.units_whole) {
+    unit = us; split = 0; nsp = 1;
+  } else {
+    const int r = us - p.units_whole;
+    unit = p.units_whole + r / p.n_splits; split = r % p.n_splits; nsp = p.n_splits;
+  }
   const int b = unit / p.Hkv, hkv = unit - b * p.Hkv;
   const int hq_in = member / p.q_tiles, qtile = member - hq_in * p.q_tiles;
   const int h = hkv * (p.H / p.Hkv) + hq_in;
@@ -167,8 +174,8 @@ __global__ void __launch_bounds__(512, 2) attn_ring8_kernel(AttnParams p) {
   };
   const int tps = p.T / BN;  // tiles per slot
   const int nt = nvis * tps;
-  const int t_begin = (int)((int64_t)split * nt / p.n_splits);
-  const int t_end = (int)((int64_t)(split + 1) * nt / p.n_splits);
+  const int t_begin = (int)((int64_t)split * nt / nsp);
+  const int t_end = (int)((int64_t)(split + 1) * nt / nsp);
   const int ntile = t_end - t_begin;
 
   // ---- Q fragments stay in registers, pre-multiplied by scale*log2(e) ----
@@ -566,13 +573,13 @@ __global__ void __launch_bounds__(512, 2) attn_ring8_kernel(AttnParams p) {
   }
 
   // ---- epilogue ----
-  const int64_t rows = (int64_t)p.B * p.H * p.T;
+  const int64_t rows = (int64_t)p.B * p.H * p.T - p.ws_row0;  // rows in the workspace
   const bool valid = qrow < p.T;
-  const float inv = (p.n_splits == 1) ? 1.f / l_tot : 1.f;
+  const float inv = (nsp == 1) ? 1.f / l_tot : 1.f;
   const int64_t row = ((int64_t)b * p.H + h) * p.T + qrow;
-  if (p.n_splits > 1 && valid && hh == 0) {
+  if (nsp > 1 && valid && hh == 0) {
     float2 ml = make_float2(m_ref, l_tot);
-    *reinterpret_cast<float2*>(p.ws_ml + ((int64_t)split * rows + row) * 2) = ml;
+    *reinterpret_cast<float2*>(p.ws_ml + ((int64_t)split * rows + (row - p.ws_row0)) * 2) = ml;
   }
 #pragma unroll
   for (int db = 0; db < DB; ++db) {
@@ -590,12 +597,12 @@ __global__ void __launch_bounds__(512, 2) attn_ring8_kernel(AttnParams p) {
       }
       const int d0 = 32 * db + 8 * (c + hh);
       if (valid) {
-        if (p.n_splits == 1) {
+        if (nsp == 1) {
           uint16_t* dst = reinterpret_cast<uint16_t*>(p.out) + b * p.os_b + h * p.os_h +
                           (int64_t)qrow * p.os_t + d0;
           *reinterpret_cast<frag_t*>(dst) = M::pack8(f[0], f[1], f[2], f[3], f[4], f[5], f[6], f[7]);
         } else {
-          float* dst = p.ws_o + ((int64_t)split * rows + row) * DH + d0;
+          float* dst = p.ws_o + ((int64_t)split * rows + (row - p.ws_row0)) * DH + d0;
           *reinterpret_cast<float4*>(dst) = make_float4(f[0], f[1], f[2], f[3]);
           *reinterpret_cast<float4*>(dst + 4) = make_float4(f[4], f[5], f[6], f[7]);
         }

@@ -22,35 +22,65 @@ int ring_shape_ok(int B, int H, int Hkv, int T, int Dh, int64_t L, int dilation)
 }
 
 struct AttnPlan {
-  int variant;   // 1: 128 queries per workgroup, 2: 256
-  int n_splits;
+  int variant;      // 1/2: 4-wavefront kernel with 128/256 queries; 3/4: 8-wavefront kernel with 128/256
+  int block_m;      // queries per workgroup
+  int n_splits;     // context splits of the units that are split (1: none)
+  int units_whole;  // leading (batch, kv head) units that are not split
+  int64_t ws_rows;  // query rows that go through the split-context workspace
 };
 
-// Pick the query-tile size and the number of context splits.  128-query workgroups (two fit per
-// CU, so softmax VALU work of one overlaps MFMA work of the other) measured faster than
-// 256-query ones at every benchmark shape.  Splits are added until the grid has one workgroup
-// per CU, but never so many that a split holds fewer than two 64-key tiles of the steady-state
-// context.
-AttnPlan plan_attn(int B, int H, int T, int64_t L, int n_splits, int variant) {
+// Pick the kernel shape and the context splitting.
+//  * Shape: the 8-wavefront kernel, 256 queries per workgroup when that alone gives at least one
+//    workgroup per CU, else 128 queries.
+//  * Few workgroups (256-token frames): every unit is split into the same number of context
+//    parts, enough for one workgroup per CU but never fewer than two 64-key tiles per part.
+//  * Many workgroups that do not divide into whole rounds of 256 CUs (e.g. 384): only the units
+//    of the last, partial round are split, so that round finishes in a fraction of the time.
+AttnPlan plan_attn(int B, int H, int Hkv, int T, int64_t L, int n_splits, int variant) {
   AttnPlan pl;
-  pl.variant = variant ? variant : 1;
+  const int64_t wg256 = (int64_t)B * H * ((T + 255) / 256);
+  pl.variant = variant ? variant : ((T >= 256 && wg256 >= 256) ? 4 : 3);
+  pl.block_m = (pl.variant == 2 || pl.variant == 4) ? 256 : 128;
+  const int units = B * Hkv;
+  const int members = (H / Hkv) * ((T + pl.block_m - 1) / pl.block_m);
+  const int64_t wgs = (int64_t)units * members;
+  const int64_t tiles = L / 64;  // visible 64-key tiles at steady state
+  const int64_t max_s = tiles / 2 > 0 ? tiles / 2 : 1;
+  pl.units_whole = 0;
+  pl.n_splits = 1;
   if (n_splits > 0) {
     pl.n_splits = n_splits;
-    return pl;
-  }
-  const int bm = (pl.variant == 2 || pl.variant == 4) ? 256 : 128;
-  const int64_t base = (int64_t)B * H * ((T + bm - 1) / bm);
-  const int64_t want = 256;
-  int s = 1;
-  if (base < want) {
-    s = (int)((want + base - 1) / base);
-    const int64_t tiles = L / 64;  // visible tiles at steady state
-    const int64_t max_s = tiles / 2 > 0 ? tiles / 2 : 1;
-    if (s > max_s) s = (int)max_s;
+  } else if (wgs < 256) {
+    int64_t s = (256 + wgs - 1) / wgs;
+    if (s > max_s) s = max_s;
     if (s > 64) s = 64;
+    pl.n_splits = (int)s;
+  } else if (wgs < 4 * 256 && members <= 256) {
+    const int whole_units = (int)((wgs / 256) * 256 / members);
+    const int64_t rem_wgs = (int64_t)(units - whole_units) * members;
+    if (rem_wgs > 0 && rem_wgs <= 128) {
+      int64_t s = 256 / rem_wgs;
+      if (s > 8) s = 8;
+      if (s > max_s / 2) s = max_s / 2;
+      if (s > 1) {
+        pl.n_splits = (int)s;
+        pl.units_whole = whole_units;
+      }
+    }
   }
-  pl.n_splits = s;
+  pl.ws_rows = pl.n_splits > 1 ? (int64_t)(units - pl.units_whole) * (H / Hkv) * T : 0;
   return pl;
+}
+
+int variant_of(int q_tile) {
+  switch (q_tile) {
+    case 0: return 0;
+    case 128: return 1;
+    case 256: return 2;
+    case 129: return 3;
+    case 257: return 4;
+    default: return -1;
+  }
 }
 
 }  // namespace
@@ -139,15 +169,18 @@ int we_rope_apply(const void* x, const int64_t x_strides[3], void* x_out, const 
 }
 
 int32_t we_attn_auto_splits(int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L) {
-  (void)Hkv; (void)Dh;
-  if (B <= 0 || H <= 0 || T <= 0 || L <= 0) return 1;
-  return plan_attn(B, H, T, L, 0, 0).n_splits;
+  (void)Dh;
+  if (B <= 0 || H <= 0 || Hkv <= 0 || H % Hkv != 0 || T <= 0 || L <= 0) return 1;
+  return plan_attn(B, H, Hkv, T, L, 0, 0).n_splits;
 }
 
-size_t we_attn_workspace_bytes(int32_t B, int32_t H, int32_t T, int32_t Dh, int32_t n_splits) {
-  if (n_splits <= 1 || B <= 0 || H <= 0 || T <= 0 || Dh <= 0) return 0;
-  const size_t rows = (size_t)B * H * T;
-  return (size_t)n_splits * rows * ((size_t)Dh + 2) * sizeof(float);
+size_t we_attn_workspace_bytes(int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L,
+                               int32_t n_splits, int32_t q_tile) {
+  if (B <= 0 || H <= 0 || Hkv <= 0 || H % Hkv != 0 || T <= 0 || Dh <= 0 || L <= 0 || n_splits < 0) return 0;
+  const int variant = variant_of(q_tile);
+  if (variant < 0) return 0;
+  const AttnPlan pl = plan_attn(B, H, Hkv, T, L, n_splits, variant);
+  return (size_t)pl.n_splits * (size_t)pl.ws_rows * ((size_t)Dh + 2) * sizeof(float);
 }
 
 int we_attn_ring_fwd(const void* q, const int64_t q_strides[3], const void* kv, const uint8_t* written,
@@ -162,34 +195,33 @@ int we_attn_ring_fwd(const void* q, const int64_t q_strides[3], const void* kv, 
   if (Dh != 64 && Dh != 128) return WE_ERR_UNSUPPORTED;
   if (T % 64 != 0 || L / T > WE_MAX_SLOTS) return WE_ERR_UNSUPPORTED;
   if (!(scale > 0.f) || n_splits < 0 || n_splits > 64) return WE_ERR_BAD_SHAPE;
-  if (q_tile != 0 && q_tile != 128 && q_tile != 256 && q_tile != 129 && q_tile != 257) return WE_ERR_UNSUPPORTED;
+  if (variant_of(q_tile) < 0) return WE_ERR_UNSUPPORTED;
   if (!aligned16(q) || !aligned16(kv) || !aligned16(out) || !strides_ok(q_strides, dtype) ||
       !strides_ok(out_strides, dtype))
     return WE_ERR_ALIGNMENT;
 
-  // 128/256: 4-wavefront kernel; 129/257: 8-wavefront LDS-DMA kernel with 128/256 queries
-  const int variant = q_tile == 0 ? 0 : (q_tile == 256 ? 2 : (q_tile == 129 ? 3 : (q_tile == 257 ? 4 : 1)));
-  const AttnPlan pl = plan_attn(B, H, T, L, n_splits, variant);
-  if (pl.n_splits > 1) {
+  const AttnPlan pl = plan_attn(B, H, Hkv, T, L, n_splits, variant_of(q_tile));
+  const size_t ws_need = (size_t)pl.n_splits * (size_t)pl.ws_rows * ((size_t)Dh + 2) * sizeof(float);
+  if (ws_need > 0) {
     if (!workspace || !aligned16(workspace)) return WE_ERR_WORKSPACE;
-    if (workspace_bytes < we_attn_workspace_bytes(B, H, T, Dh, pl.n_splits)) return WE_ERR_WORKSPACE;
+    if (workspace_bytes < ws_need) return WE_ERR_WORKSPACE;
   }
 
   we::AttnParams p;
   p.q = q; p.kv = kv; p.written = written; p.t_pos = t_pos; p.out = out;
-  const size_t rows = (size_t)B * H * T;
-  p.ws_o = static_cast<float*>(workspace);
-  p.ws_ml = p.ws_o ? p.ws_o + (size_t)pl.n_splits * rows * Dh : nullptr;
+  p.ws_o = ws_need ? static_cast<float*>(workspace) : nullptr;
+  p.ws_ml = ws_need ? p.ws_o + (size_t)pl.n_splits * (size_t)pl.ws_rows * Dh : nullptr;
   p.qs_b = q_strides[0]; p.qs_h = q_strides[1]; p.qs_t = q_strides[2];
   p.os_b = out_strides[0]; p.os_h = out_strides[1]; p.os_t = out_strides[2];
   p.L = L;
   p.B = B; p.H = H; p.Hkv = Hkv; p.T = T;
   p.n_slots = (int)(L / T); p.dilation = dilation; p.num_buckets = p.n_slots / dilation;
   p.n_splits = pl.n_splits;
-  const int bm = (pl.variant == 2 || pl.variant == 4) ? 256 : 128;
-  p.q_tiles = (T + bm - 1) / bm;
+  p.units_whole = pl.units_whole;
+  p.ws_row0 = (int64_t)B * H * T - pl.ws_rows;
+  p.q_tiles = (T + pl.block_m - 1) / pl.block_m;
   p.members = (H / Hkv) * p.q_tiles;
-  p.unit_splits = B * Hkv * pl.n_splits;
+  p.unit_splits = pl.units_whole + (B * Hkv - pl.units_whole) * pl.n_splits;
   p.scale_log2 = scale * 1.4426950408889634f;
 
   hipStream_t st = static_cast<hipStream_t>(stream);

@@ -35,24 +35,25 @@ struct AttnParams {
   const uint8_t* written;
   const int64_t* t_pos;
   void* out;
-  float* ws_o;   // [n_splits][B*H*T][Dh] unnormalised partial outputs
-  float* ws_ml;  // [n_splits][B*H*T][2]  running max (log2 domain) and sum
+  float* ws_o;   // [n_splits][rows >= ws_row0][Dh] unnormalised partial outputs
+  float* ws_ml;  // [n_splits][rows >= ws_row0][2]  running max (log2 domain) and sum
   int64_t qs_b, qs_h, qs_t;
   int64_t os_b, os_h, os_t;
   int64_t L;
   int B, H, Hkv, T;
   int n_slots, dilation, num_buckets;
-  int n_splits;
+  int n_splits;     // context splits of the units that are split (1 = nothing is split)
+  int units_whole;  // leading (batch, kv head) units processed unsplit, writing the output directly
+  int64_t ws_row0;  // first query row covered by the split-context workspace
   int q_tiles;      // ceil(T / queries per workgroup)
   int members;      // workgroups that share one K/V stream: (H/Hkv) * q_tiles
-  int unit_splits;  // B * Hkv * n_splits
+  int unit_splits;  // units_whole + (B * Hkv - units_whole) * n_splits
   float scale_log2; // softmax scale * log2(e)
 };
 
 hipError_t launch_rope_kv_store(const StoreParams& p, int dtype, hipStream_t stream);
 
-// queries handled by one workgroup of the attention kernel for a head dim / variant
-int attn_block_m(int Dh, int variant);
+// 4-wavefront kernel: variant 1 -> 128 queries per workgroup, 2 -> 256
 hipError_t launch_attn_ring(const AttnParams& p, int Dh, int dtype, int variant, hipStream_t stream);
 // 8-wavefront LDS-DMA kernel: groups = 2 -> 128 queries per workgroup, 1 -> 256
 hipError_t launch_attn_ring8(const AttnParams& p, int Dh, int dtype, int groups, hipStream_t stream);

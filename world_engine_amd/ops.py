@@ -146,8 +146,10 @@ def attn_auto_splits(B: int, H: int, Hkv: int, T: int, Dh: int, L: int) -> int:
     return int(_capi.lib().we_attn_auto_splits(B, H, Hkv, T, Dh, L))
 
 
-def attn_workspace_bytes(B: int, H: int, T: int, Dh: int, n_splits: int) -> int:
-    return int(_capi.lib().we_attn_workspace_bytes(B, H, T, Dh, n_splits))
+def attn_workspace_bytes(B: int, H: int, Hkv: int, T: int, Dh: int, L: int, n_splits: int = 0,
+                         q_tile: int = 0) -> int:
+    """Bytes of split-context workspace ``attn_ring`` needs for these sizes and knobs."""
+    return int(_capi.lib().we_attn_workspace_bytes(B, H, Hkv, T, Dh, L, n_splits, q_tile))
 
 
 def attn_ring(q: Tensor, kv: Tensor, written: Tensor, t_pos: Tensor, L: int, dilation: int,
@@ -177,11 +179,7 @@ def attn_ring(q: Tensor, kv: Tensor, written: Tensor, t_pos: Tensor, L: int, dil
         raise RuntimeError("t_pos must be a non-empty int64 tensor")
     scale = 1.0 / math.sqrt(Dh) if scale is None else float(scale)
     lib = _capi.lib()
-    if n_splits == 0:
-        n_eff = int(lib.we_attn_auto_splits(B, H, Hkv, T, Dh, L))
-    else:
-        n_eff = n_splits
-    ws_bytes = int(lib.we_attn_workspace_bytes(B, H, T, Dh, n_eff))
+    ws_bytes = int(lib.we_attn_workspace_bytes(B, H, Hkv, T, Dh, L, n_splits, q_tile))
     if ws_bytes and (workspace is None or workspace.numel() * workspace.element_size() < ws_bytes):
         workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     if out is None:
@@ -196,7 +194,7 @@ def attn_ring(q: Tensor, kv: Tensor, written: Tensor, t_pos: Tensor, L: int, dil
         out.data_ptr(), _bhtd_strides(out, "out"),
         workspace.data_ptr() if ws_bytes else None,
         workspace.numel() * workspace.element_size() if ws_bytes else 0,
-        B, H, Hkv, T, Dh, L, dilation, scale, n_eff, q_tile, _dtype_code(q), _stream_ptr(dev))
+        B, H, Hkv, T, Dh, L, dilation, scale, n_splits, q_tile, _dtype_code(q), _stream_ptr(dev))
     _capi.check(code, "we_attn_ring_fwd")
     return out
 
