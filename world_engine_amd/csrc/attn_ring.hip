@@ -393,7 +393,7 @@ __global__ void __launch_bounds__(256, NQB == 1 ? 2 : 1) attn_ring_kernel(AttnPa
     half_wave_pair(l_run[qb], lo, up);
     const float l_tot = lo + up;
     const bool valid = qrow[qb] < p.T;
-    const float inv = (nsp == 1) ? 1.f / l_tot : 1.f;
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     const int64_t row = ((int64_t)b * p.H + h) * p.T + qrow[qb];
     if (nsp > 1 && valid && hh == 0) {
       float2 ml = make_float2(m_run[qb], l_tot);
@@ -421,9 +421,8 @@ __global__ void __launch_bounds__(256, NQB == 1 ? 2 : 1) attn_ring_kernel(AttnPa
                             (int64_t)qrow[qb] * p.os_t + d0;
             *reinterpret_cast<frag_t*>(dst) = M::pack8(f[0], f[1], f[2], f[3], f[4], f[5], f[6], f[7]);
           } else {
-            float* dst = p.ws_o + ((int64_t)split * rows + (row - p.ws_row0)) * DH + d0;
-            *reinterpret_cast<float4*>(dst) = make_float4(f[0], f[1], f[2], f[3]);
-            *reinterpret_cast<float4*>(dst + 4) = make_float4(f[4], f[5], f[6], f[7]);
+            uint16_t* dst = p.ws_o + ((int64_t)split * rows + (row - p.ws_row0)) * DH + d0;
+            *reinterpret_cast<frag_t*>(dst) = M::pack8(f[0], f[1], f[2], f[3], f[4], f[5], f[6], f[7]);
           }
         }
       }
@@ -431,28 +430,30 @@ __global__ void __launch_bounds__(256, NQB == 1 ? 2 : 1) attn_ring_kernel(AttnPa
   }
 }
 
-// Second pass of the split-context path: out = sum_s w_s O_s / sum_s w_s l_s with
-// w_s = 2^(m_s - max_s m_s).  One thread per (query row, 4 head-dim columns).
+// Second pass of the split-context path.  Every split left, per query row, its normalised
+// output O_s (element type), its reference m_s (log2 domain) and its sum l_s; the result is
+// sum_s w_s O_s / sum_s w_s with w_s = 2^(m_s - max m) * l_s.  One thread per (row, 8 columns).
 template <typename M, int DH>
 __global__ void __launch_bounds__(256) attn_combine_kernel(AttnParams p) {
+  typedef typename M::frag_t frag_t;
   const int64_t rows = (int64_t)p.B * p.H * p.T - p.ws_row0;  // rows that were split
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= rows * (DH / 4)) return;
-  const int64_t row = idx / (DH / 4);  // workspace row; query row = row + ws_row0
-  const int dg = (int)(idx % (DH / 4));
+  if (idx >= rows * (DH / 8)) return;
+  const int64_t row = idx / (DH / 8);  // workspace row; query row = row + ws_row0
+  const int dg = (int)(idx % (DH / 8));
   float mmax = -INFINITY;
   for (int s = 0; s < p.n_splits; ++s) mmax = fmaxf(mmax, p.ws_ml[((int64_t)s * rows + row) * 2]);
   float den = 0.f;
-  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  float acc[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) acc[j] = 0.f;
   for (int s = 0; s < p.n_splits; ++s) {
     const float2 ml = *reinterpret_cast<const float2*>(p.ws_ml + ((int64_t)s * rows + row) * 2);
-    const float w = __builtin_amdgcn_exp2f(ml.x - mmax);
-    const float4 ov = *reinterpret_cast<const float4*>(p.ws_o + ((int64_t)s * rows + row) * DH + dg * 4);
-    den += w * ml.y;
-    acc.x += w * ov.x;
-    acc.y += w * ov.y;
-    acc.z += w * ov.z;
-    acc.w += w * ov.w;
+    const float w = __builtin_amdgcn_exp2f(ml.x - mmax) * ml.y;
+    const frag_t ov = *reinterpret_cast<const frag_t*>(p.ws_o + ((int64_t)s * rows + row) * DH + dg * 8);
+    den += w;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] += w * (float)ov[j];
   }
   const float inv = 1.f / den;
   const int64_t qrow = row + p.ws_row0;
@@ -460,10 +461,9 @@ __global__ void __launch_bounds__(256) attn_combine_kernel(AttnParams p) {
   const int64_t bh = qrow / p.T;
   const int h = (int)(bh % p.H);
   const int b = (int)(bh / p.H);
-  uint16_t* dst = reinterpret_cast<uint16_t*>(p.out) + b * p.os_b + h * p.os_h + (int64_t)t * p.os_t + dg * 4;
-  typename M::frag_t pk = M::pack8(acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv, 0.f, 0.f, 0.f, 0.f);
-  const uint4 bits = __builtin_bit_cast(uint4, pk);
-  *reinterpret_cast<uint2*>(dst) = make_uint2(bits.x, bits.y);
+  uint16_t* dst = reinterpret_cast<uint16_t*>(p.out) + b * p.os_b + h * p.os_h + (int64_t)t * p.os_t + dg * 8;
+  *reinterpret_cast<frag_t*>(dst) = M::pack8(acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv, acc[4] * inv,
+                                             acc[5] * inv, acc[6] * inv, acc[7] * inv);
 }
 
 template <typename M, int DH, int NQB>
@@ -495,7 +495,7 @@ hipError_t launch_attn_ring(const AttnParams& p, int Dh, int dtype, int variant,
 }
 
 hipError_t launch_attn_combine(const AttnParams& p, int Dh, int dtype, hipStream_t stream) {
-  const int64_t total = ((int64_t)p.B * p.H * p.T - p.ws_row0) * (Dh / 4);
+  const int64_t total = ((int64_t)p.B * p.H * p.T - p.ws_row0) * (Dh / 8);
   const unsigned grid = (unsigned)((total + 255) / 256);
   if (dtype == WE_DTYPE_BF16) {
     if (Dh == 128) hipLaunchKernelGGL((attn_combine_kernel<Bf16Mma, 128>), dim3(grid), dim3(256), 0, stream, p);

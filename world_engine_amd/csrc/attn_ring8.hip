@@ -138,6 +138,17 @@ __global__ void __launch_bounds__(512, 2) attn_ring8_kernel(AttnParams p) {
   const int hq_in = member / p.q_tiles, qtile = member - hq_in * p.q_tiles;
   const int h = hkv * (p.H / p.Hkv) + hq_in;
 
+  // ---- raw Q fragments: requested first so the loads overlap the slot-list construction ----
+  frag_t qf[KS];
+  const int qrow = qtile * BM + qb * 32 + l32;
+  {
+    const uint16_t* qbase = reinterpret_cast<const uint16_t*>(p.q) + b * p.qs_b + h * p.qs_h;
+    const int qr = qrow < p.T ? qrow : p.T - 1;
+    const uint16_t* src = qbase + (int64_t)qr * p.qs_t + hh * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = *reinterpret_cast<const frag_t*>(src + ks * 16);
+  }
+
   // ---- list of visible slots (the tail is pseudo-slot n_slots) ----
   if (wave == 0) {
     const SlotInfo si = ring_slot(p.t_pos[0], p.dilation, p.num_buckets);
@@ -178,20 +189,13 @@ __global__ void __launch_bounds__(512, 2) attn_ring8_kernel(AttnParams p) {
   const int t_end = (int)((int64_t)(split + 1) * nt / nsp);
   const int ntile = t_end - t_begin;
 
-  // ---- Q fragments stay in registers, pre-multiplied by scale*log2(e) ----
+  // ---- Q stays in registers for the whole kernel, pre-multiplied by scale*log2(e) ----
   const float c2 = p.scale_log2;
-  frag_t qf[KS];
-  const int qrow = qtile * BM + qb * 32 + l32;
-  {
-    const uint16_t* qbase = reinterpret_cast<const uint16_t*>(p.q) + b * p.qs_b + h * p.qs_h;
-    const int qr = qrow < p.T ? qrow : p.T - 1;
-    const uint16_t* src = qbase + (int64_t)qr * p.qs_t + hh * 8;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const frag_t raw = *reinterpret_cast<const frag_t*>(src + ks * 16);
-      qf[ks] = M::pack8((float)raw[0] * c2, (float)raw[1] * c2, (float)raw[2] * c2, (float)raw[3] * c2,
-                        (float)raw[4] * c2, (float)raw[5] * c2, (float)raw[6] * c2, (float)raw[7] * c2);
-    }
+  for (int ks = 0; ks < KS; ++ks) {
+    const frag_t raw = qf[ks];
+    qf[ks] = M::pack8((float)raw[0] * c2, (float)raw[1] * c2, (float)raw[2] * c2, (float)raw[3] * c2,
+                      (float)raw[4] * c2, (float)raw[5] * c2, (float)raw[6] * c2, (float)raw[7] * c2);
   }
 
   const int64_t cap = p.L + p.T;
@@ -227,23 +231,21 @@ __global__ void __launch_bounds__(512, 2) attn_ring8_kernel(AttnParams p) {
       }
     }
   };
-  auto tile_base = [&](uint64_t base, const TileWalk& w) __attribute__((always_inline)) {
-    const int slot = vis_at(w.sidx);
-    const int64_t row0 = (int64_t)slot * p.T + (int64_t)w.sub * BN;
-    return uniform64(base + (uint64_t)row0 * ROW_B);
+  // byte offset of a tile inside its (batch, kv head) plane; fits 32 bits (checked on the host)
+  auto tile_off = [&](const TileWalk& w) __attribute__((always_inline)) {
+    return (uint32_t)(vis_at(w.sidx) * p.T + w.sub * BN) * (uint32_t)ROW_B;
   };
-  auto dma_tile = [&](uint64_t base, const uint32_t(&voff)[NDMA], const TileWalk& w, uint32_t lds_tile)
-                      __attribute__((always_inline)) {
-    const uint64_t g = tile_base(base, w);
+  const uint64_t kplane = uniform64(kbase), vplane = uniform64(vbase);
+  auto dma_k = [&](uint32_t off, int slot) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < NDMA; ++i)
-      dma16(g, voff[i], __builtin_amdgcn_readfirstlane(lds_tile + (wave + i * 8) * 1024));
+      dma16(kplane, kvoff[i] + off, __builtin_amdgcn_readfirstlane(lds0 + slot * TILE_B + (wave + i * 8) * 1024));
   };
-  auto dma_k = [&](const TileWalk& w, int slot) __attribute__((always_inline)) {
-    dma_tile(kbase, kvoff, w, lds0 + slot * TILE_B);
-  };
-  auto dma_v = [&](const TileWalk& w, int slot) __attribute__((always_inline)) {
-    dma_tile(vbase, vvoff, w, lds0 + L::V_OFF + slot * TILE_B);
+  auto dma_v = [&](uint32_t off, int slot) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < NDMA; ++i)
+      dma16(vplane, vvoff[i] + off,
+            __builtin_amdgcn_readfirstlane(lds0 + L::V_OFF + slot * TILE_B + (wave + i * 8) * 1024));
   };
 
   // ---- fragment read addresses (byte offsets into smem) ----
@@ -450,13 +452,27 @@ __global__ void __launch_bounds__(512, 2) attn_ring8_kernel(AttnParams p) {
     // block per tile and prefetches its next fragments across the barrier); the prologue issues
     // what the iterations before 0 would have.
     constexpr int KA = KSPLIT == 1 ? 3 : 4;
-    TileWalk kw = walk_init(), vw = walk_init();
-    dma_k(kw, 0); walk_next(kw);
-    dma_k(kw, 1); walk_next(kw);
-    if (KSPLIT == 2) { dma_k(kw, 2); walk_next(kw); }
-    dma_v(vw, 0); walk_next(vw);
-    dma_k(kw, KA - 1); walk_next(kw);
-    dma_v(vw, 1); walk_next(vw);
+    // The V stream trails the K stream by KA - 2 tiles, so it reuses the K stream's offsets.
+    TileWalk kw = walk_init();
+    uint32_t off1, off2;  // offsets of the last and the last-but-one tile the K stream visited
+    {
+      const uint32_t o0 = tile_off(kw); walk_next(kw);
+      const uint32_t o1 = tile_off(kw); walk_next(kw);
+      const uint32_t o2 = tile_off(kw); walk_next(kw);
+      dma_k(o0, 0);
+      dma_k(o1, 1);
+      if (KSPLIT == 2) dma_k(o2, 2);
+      dma_v(o0, 0);
+      if (KSPLIT == 1) {
+        dma_k(o2, 2);
+        off1 = o2; off2 = o1;
+      } else {
+        const uint32_t o3 = tile_off(kw); walk_next(kw);
+        dma_k(o3, 3);
+        off1 = o3; off2 = o2;
+      }
+      dma_v(o1, 1);
+    }
     dma_wait<(KA + 1) * NDMA>();
     __syncthreads();  // K(0) and the zeroed V slot are in LDS
     // first block: plain logits, reference = its row max, shifted by hand
@@ -482,10 +498,12 @@ __global__ void __launch_bounds__(512, 2) attn_ring8_kernel(AttnParams p) {
     auto iteration = [&](int j, auto jm_c) __attribute__((always_inline)) {
       constexpr int JM = decltype(jm_c)::value;
       auto issue_dma = [&]() __attribute__((always_inline)) {
-        dma_k(kw, (JM + KA) % NST);  // K(j+KA)
+        const uint32_t o = tile_off(kw);
         walk_next(kw);
-        dma_v(vw, (JM + 2) % NST);   // V(j+2)
-        walk_next(vw);
+        dma_k(o, (JM + KA) % NST);                       // K(j+KA)
+        dma_v(KA == 3 ? off1 : off2, (JM + 2) % NST);    // V(j+2)
+        off2 = off1;
+        off1 = o;
       };
       auto nothing = [&]() __attribute__((always_inline)) {};
       if (KSPLIT == 1) {
@@ -575,7 +593,7 @@ __global__ void __launch_bounds__(512, 2) attn_ring8_kernel(AttnParams p) {
   // ---- epilogue ----
   const int64_t rows = (int64_t)p.B * p.H * p.T - p.ws_row0;  // rows in the workspace
   const bool valid = qrow < p.T;
-  const float inv = (nsp == 1) ? 1.f / l_tot : 1.f;
+  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   const int64_t row = ((int64_t)b * p.H + h) * p.T + qrow;
   if (nsp > 1 && valid && hh == 0) {
     float2 ml = make_float2(m_ref, l_tot);
@@ -602,9 +620,8 @@ __global__ void __launch_bounds__(512, 2) attn_ring8_kernel(AttnParams p) {
                           (int64_t)qrow * p.os_t + d0;
           *reinterpret_cast<frag_t*>(dst) = M::pack8(f[0], f[1], f[2], f[3], f[4], f[5], f[6], f[7]);
         } else {
-          float* dst = p.ws_o + ((int64_t)split * rows + (row - p.ws_row0)) * DH + d0;
-          *reinterpret_cast<float4*>(dst) = make_float4(f[0], f[1], f[2], f[3]);
-          *reinterpret_cast<float4*>(dst + 4) = make_float4(f[4], f[5], f[6], f[7]);
+          uint16_t* dst = p.ws_o + ((int64_t)split * rows + (row - p.ws_row0)) * DH + d0;
+          *reinterpret_cast<frag_t*>(dst) = M::pack8(f[0], f[1], f[2], f[3], f[4], f[5], f[6], f[7]);
         }
       }
     }

@@ -180,7 +180,7 @@ size_t we_attn_workspace_bytes(int32_t B, int32_t H, int32_t Hkv, int32_t T, int
   const int variant = variant_of(q_tile);
   if (variant < 0) return 0;
   const AttnPlan pl = plan_attn(B, H, Hkv, T, L, n_splits, variant);
-  return (size_t)pl.n_splits * (size_t)pl.ws_rows * ((size_t)Dh + 2) * sizeof(float);
+  return (size_t)pl.n_splits * (size_t)pl.ws_rows * ((size_t)Dh * 2 + 2 * sizeof(float));
 }
 
 int we_attn_ring_fwd(const void* q, const int64_t q_strides[3], const void* kv, const uint8_t* written,
@@ -194,6 +194,7 @@ int we_attn_ring_fwd(const void* q, const int64_t q_strides[3], const void* kv, 
   if (dtype != WE_DTYPE_BF16 && dtype != WE_DTYPE_F16) return WE_ERR_UNSUPPORTED;
   if (Dh != 64 && Dh != 128) return WE_ERR_UNSUPPORTED;
   if (T % 64 != 0 || L / T > WE_MAX_SLOTS) return WE_ERR_UNSUPPORTED;
+  if ((uint64_t)(L + T) * (uint64_t)Dh * 2u >= (1ull << 32)) return WE_ERR_UNSUPPORTED;  // 32-bit tile offsets
   if (!(scale > 0.f) || n_splits < 0 || n_splits > 64) return WE_ERR_BAD_SHAPE;
   if (variant_of(q_tile) < 0) return WE_ERR_UNSUPPORTED;
   if (!aligned16(q) || !aligned16(kv) || !aligned16(out) || !strides_ok(q_strides, dtype) ||
@@ -201,7 +202,7 @@ int we_attn_ring_fwd(const void* q, const int64_t q_strides[3], const void* kv, 
     return WE_ERR_ALIGNMENT;
 
   const AttnPlan pl = plan_attn(B, H, Hkv, T, L, n_splits, variant_of(q_tile));
-  const size_t ws_need = (size_t)pl.n_splits * (size_t)pl.ws_rows * ((size_t)Dh + 2) * sizeof(float);
+  const size_t ws_need = (size_t)pl.n_splits * (size_t)pl.ws_rows * ((size_t)Dh * 2 + 2 * sizeof(float));
   if (ws_need > 0) {
     if (!workspace || !aligned16(workspace)) return WE_ERR_WORKSPACE;
     if (workspace_bytes < ws_need) return WE_ERR_WORKSPACE;
@@ -209,8 +210,8 @@ int we_attn_ring_fwd(const void* q, const int64_t q_strides[3], const void* kv, 
 
   we::AttnParams p;
   p.q = q; p.kv = kv; p.written = written; p.t_pos = t_pos; p.out = out;
-  p.ws_o = ws_need ? static_cast<float*>(workspace) : nullptr;
-  p.ws_ml = ws_need ? p.ws_o + (size_t)pl.n_splits * (size_t)pl.ws_rows * Dh : nullptr;
+  p.ws_o = ws_need ? static_cast<uint16_t*>(workspace) : nullptr;
+  p.ws_ml = ws_need ? reinterpret_cast<float*>(p.ws_o + (size_t)pl.n_splits * (size_t)pl.ws_rows * Dh) : nullptr;
   p.qs_b = q_strides[0]; p.qs_h = q_strides[1]; p.qs_t = q_strides[2];
   p.os_b = out_strides[0]; p.os_h = out_strides[1]; p.os_t = out_strides[2];
   p.L = L;

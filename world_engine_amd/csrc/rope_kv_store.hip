@@ -6,7 +6,7 @@
 // The ring slot is derived on the device from t_pos[0] (:126-131,:140).
 //
 // Work item: one thread per 16 consecutive input elements of one (tensor, b, head, token)
-// row.  For a rotated row those are 8 (even, odd) pairs; the thread writes 8 contiguous
+// row; a workgroup covers 256 consecutive (token, chunk) pairs of one head.  For a rotated row those are 8 (even, odd) pairs; the thread writes 8 contiguous
 // elements into the first half of the output row and 8 into the second half (the reference
 // concatenates the rotated halves, attn.py:40).  Threads are ordered chunk-fastest, then
 // token, so a wavefront reads whole 256-byte input rows and writes contiguous cache rows.
@@ -77,20 +77,17 @@ __device__ __forceinline__ void store8(void* p, const Chunk8<Tag>& c) {
 template <typename Tag>
 __global__ void __launch_bounds__(256) rope_kv_store_kernel(StoreParams p) {
   typedef typename Tag::store_t st_t;
+  // grid: x = 256-thread slices of the (token, chunk) pairs of one row block, y = head among
+  // [q heads | k heads | v heads], z = batch; everything below the block level is 32-bit math
   const int cpr = p.Dh >> 4;  // 16-element chunks per row
   const int hq = p.q ? p.H : 0;
   const int hkv = p.k ? p.Hkv : 0;  // rotation-only launches carry no k/v
-  const int heads_all = hq + 2 * hkv;
-  const int64_t total = (int64_t)p.B * heads_all * p.T * cpr;
-  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx >= total) return;
-
-  const int chunk = (int)(idx % cpr);
-  int64_t row = idx / cpr;
-  const int t = (int)(row % p.T);
-  row /= p.T;
-  const int head_all = (int)(row % heads_all);
-  const int b = (int)(row / heads_all);
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= p.T * cpr) return;
+  const int t = idx / cpr;
+  const int chunk = idx - t * cpr;
+  const int head_all = blockIdx.y;
+  const int b = blockIdx.z;
 
   // which tensor this row belongs to: 0 = q, 1 = k, 2 = v
   int which, h;
@@ -187,14 +184,13 @@ __global__ void __launch_bounds__(256) rope_kv_store_kernel(StoreParams p) {
 hipError_t launch_rope_kv_store(const StoreParams& p, int dtype, hipStream_t stream) {
   const int hq = p.q ? p.H : 0;
   const int hkv = p.k ? p.Hkv : 0;
-  const int64_t total = (int64_t)p.B * (hq + 2 * hkv) * p.T * (p.Dh >> 4);
-  const unsigned grid = (unsigned)((total + 255) / 256);
+  const dim3 grid((unsigned)((p.T * (p.Dh >> 4) + 255) / 256), (unsigned)(hq + 2 * hkv), (unsigned)p.B);
   if (dtype == 0)
-    hipLaunchKernelGGL(rope_kv_store_kernel<Bf16Tag>, dim3(grid), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL(rope_kv_store_kernel<Bf16Tag>, grid, dim3(256), 0, stream, p);
   else if (dtype == 1)
-    hipLaunchKernelGGL(rope_kv_store_kernel<F16Tag>, dim3(grid), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL(rope_kv_store_kernel<F16Tag>, grid, dim3(256), 0, stream, p);
   else
-    hipLaunchKernelGGL(rope_kv_store_kernel<F32Tag>, dim3(grid), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL(rope_kv_store_kernel<F32Tag>, grid, dim3(256), 0, stream, p);
   return hipGetLastError();
 }
 

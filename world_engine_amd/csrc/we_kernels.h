@@ -35,8 +35,8 @@ struct AttnParams {
   const uint8_t* written;
   const int64_t* t_pos;
   void* out;
-  float* ws_o;   // [n_splits][rows >= ws_row0][Dh] unnormalised partial outputs
-  float* ws_ml;  // [n_splits][rows >= ws_row0][2]  running max (log2 domain) and sum
+  uint16_t* ws_o;  // [n_splits][rows >= ws_row0][Dh] normalised partial outputs, element type
+  float* ws_ml;    // [n_splits][rows >= ws_row0][2]  softmax reference (log2 domain) and sum
   int64_t qs_b, qs_h, qs_t;
   int64_t os_b, os_h, os_t;
   int64_t L;
