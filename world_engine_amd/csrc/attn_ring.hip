@@ -441,19 +441,36 @@ __global__ void __launch_bounds__(256) attn_combine_kernel(AttnParams p) {
   if (idx >= rows * (DH / 8)) return;
   const int64_t row = idx / (DH / 8);  // workspace row; query row = row + ws_row0
   const int dg = (int)(idx % (DH / 8));
-  float mmax = -INFINITY;
-  for (int s = 0; s < p.n_splits; ++s) mmax = fmaxf(mmax, p.ws_ml[((int64_t)s * rows + row) * 2]);
-  float den = 0.f;
+  // Splits are merged eight at a time with all sixteen loads of a batch issued before the first
+  // use (a plain loop over a run-time split count would serialise one memory round trip per split).
+  float mmax = -INFINITY, den = 0.f;
   float acc[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) acc[j] = 0.f;
-  for (int s = 0; s < p.n_splits; ++s) {
-    const float2 ml = *reinterpret_cast<const float2*>(p.ws_ml + ((int64_t)s * rows + row) * 2);
-    const float w = __builtin_amdgcn_exp2f(ml.x - mmax) * ml.y;
-    const frag_t ov = *reinterpret_cast<const frag_t*>(p.ws_o + ((int64_t)s * rows + row) * DH + dg * 8);
-    den += w;
+  for (int s0 = 0; s0 < p.n_splits; s0 += 8) {
+    float2 ml[8];
+    frag_t ov[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[j] += w * (float)ov[j];
+    for (int j = 0; j < 8; ++j) {
+      const int s = s0 + j < p.n_splits ? s0 + j : p.n_splits - 1;  // clamp: duplicates get weight 0 below
+      ml[j] = *reinterpret_cast<const float2*>(p.ws_ml + ((int64_t)s * rows + row) * 2);
+      ov[j] = *reinterpret_cast<const frag_t*>(p.ws_o + ((int64_t)s * rows + row) * DH + dg * 8);
+    }
+    float bmax = mmax;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) bmax = fmaxf(bmax, ml[j].x);
+    const float carry = bmax > -INFINITY ? __builtin_amdgcn_exp2f(mmax - bmax) : 0.f;  // 0 on the first batch
+    den *= carry;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] *= carry;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float w = (s0 + j < p.n_splits && ml[j].y > 0.f) ? __builtin_amdgcn_exp2f(ml[j].x - bmax) * ml[j].y : 0.f;
+      den += w;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += w * (float)ov[j][e];
+    }
+    mmax = bmax;
   }
   const float inv = 1.f / den;
   const int64_t qrow = row + p.ws_row0;

@@ -112,6 +112,7 @@ __global__ void __launch_bounds__(256) rope_kv_store_kernel(StoreParams p) {
 
   Chunk16<Tag> in;
   load16<Tag>(in, src + chunk * 16);
+  const int64_t frame_t = p.t_pos[0];  // requested together with the row, used only for k/v rows
 
   const bool rotate = (which != 2) && (p.cos_t != nullptr);
   Chunk8<Tag> lo, hi;  // outputs for [8*chunk, 8*chunk+8) and [Dh/2 + 8*chunk, ...)
@@ -155,7 +156,7 @@ __global__ void __launch_bounds__(256) rope_kv_store_kernel(StoreParams p) {
 
   // K or V row: tail always, ring slot when this is an unfrozen persisting frame.
   const int64_t cap = p.L + p.T;
-  const SlotInfo si = ring_slot(p.t_pos[0], p.dilation, p.num_buckets);
+  const SlotInfo si = ring_slot(frame_t, p.dilation, p.num_buckets);
   const int plane = which - 1;
   st_t* plane_base = (st_t*)p.kv + (((int64_t)plane * p.B + b) * p.Hkv + h) * cap * p.Dh;
   const bool to_ring = (!p.frozen) && si.write_step;
