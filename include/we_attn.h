@@ -136,9 +136,7 @@ size_t we_attn_workspace_bytes(int32_t B, int32_t H, int32_t Hkv, int32_t T, int
  *                        of workgroups: only that round's units are split); 1 = single pass;
  *                        2..64 = split the visible context of every unit into that many parts.
  *                        Split parts are combined by a second kernel.
- *   q_tile               kernel shape: 0 = choose automatically; 129 / 257 = 8-wavefront
- *                        LDS-DMA kernel with 128 / 256 queries per workgroup; 128 / 256 =
- *                        4-wavefront register-staged kernel with 128 / 256 queries.
+ *   q_tile               queries per workgroup: 0 = choose automatically, or 128 / 256.
  *   scale                softmax scale (> 0); the reference uses 1/sqrt(Dh).
  *
  * Requirements: dtype bf16 or f16; Dh in {64, 128}; T % 64 == 0; L/T <= WE_MAX_SLOTS;

@@ -1,0 +1,77 @@
+// Second pass of split-context attention over the KV ring buffer (gfx950): merges the per-split
+// partial results the main kernel (attn_ring.hip) leaves in the workspace.
+// HBM-bound: reads n_splits * (Dh * 2 + 8) bytes and writes Dh * 2 bytes per query row that was
+// split.
+#include "attn_mma.h"
+#include "we_kernels.h"
+#include "../../include/we_attn.h"
+
+namespace we {
+
+// Second pass of the split-context path.  Every split left, per query row, its normalised
+// output O_s (element type), its reference m_s (log2 domain) and its sum l_s; the result is
+// sum_s w_s O_s / sum_s w_s with w_s = 2^(m_s - max m) * l_s.  One thread per (row, 8 columns).
+template <typename M, int DH>
+__global__ void __launch_bounds__(256) attn_combine_kernel(AttnParams p) {
+  typedef typename M::frag_t frag_t;
+  const int64_t rows = (int64_t)p.B * p.H * p.T - p.ws_row0;  // rows that were split
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= rows * (DH / 8)) return;
+  const int64_t row = idx / (DH / 8);  // workspace row; query row = row + ws_row0
+  const int dg = (int)(idx % (DH / 8));
+  // Splits are merged eight at a time with all sixteen loads of a batch issued before the first
+  // use (a plain loop over a run-time split count would serialise one memory round trip per split).
+  float mmax = -INFINITY, den = 0.f;
+  float acc[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+  for (int s0 = 0; s0 < p.n_splits; s0 += 8) {
+    float2 ml[8];
+    frag_t ov[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int s = s0 + j < p.n_splits ? s0 + j : p.n_splits - 1;  // clamp: duplicates get weight 0 below
+      ml[j] = *reinterpret_cast<const float2*>(p.ws_ml + ((int64_t)s * rows + row) * 2);
+      ov[j] = *reinterpret_cast<const frag_t*>(p.ws_o + ((int64_t)s * rows + row) * DH + dg * 8);
+    }
+    float bmax = mmax;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) bmax = fmaxf(bmax, ml[j].x);
+    const float carry = bmax > -INFINITY ? __builtin_amdgcn_exp2f(mmax - bmax) : 0.f;  // 0 on the first batch
+    den *= carry;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] *= carry;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float w = (s0 + j < p.n_splits && ml[j].y > 0.f) ? __builtin_amdgcn_exp2f(ml[j].x - bmax) * ml[j].y : 0.f;
+      den += w;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += w * (float)ov[j][e];
+    }
+    mmax = bmax;
+  }
+  const float inv = 1.f / den;
+  const int64_t qrow = row + p.ws_row0;
+  const int t = (int)(qrow % p.T);
+  const int64_t bh = qrow / p.T;
+  const int h = (int)(bh % p.H);
+  const int b = (int)(bh / p.H);
+  uint16_t* dst = reinterpret_cast<uint16_t*>(p.out) + b * p.os_b + h * p.os_h + (int64_t)t * p.os_t + dg * 8;
+  *reinterpret_cast<frag_t*>(dst) = M::pack8(acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv, acc[4] * inv,
+                                             acc[5] * inv, acc[6] * inv, acc[7] * inv);
+}
+
+hipError_t launch_attn_combine(const AttnParams& p, int Dh, int dtype, hipStream_t stream) {
+  const int64_t total = ((int64_t)p.B * p.H * p.T - p.ws_row0) * (Dh / 8);
+  const unsigned grid = (unsigned)((total + 255) / 256);
+  if (dtype == WE_DTYPE_BF16) {
+    if (Dh == 128) hipLaunchKernelGGL((attn_combine_kernel<Bf16Mma, 128>), dim3(grid), dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL((attn_combine_kernel<Bf16Mma, 64>), dim3(grid), dim3(256), 0, stream, p);
+  } else {
+    if (Dh == 128) hipLaunchKernelGGL((attn_combine_kernel<F16Mma, 128>), dim3(grid), dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL((attn_combine_kernel<F16Mma, 64>), dim3(grid), dim3(256), 0, stream, p);
+  }
+  return hipGetLastError();
+}
+
+}  // namespace we

@@ -1,4 +1,5 @@
-// Frame-block-causal flash attention over the KV ring buffer (gfx950, wave64, MFMA).
+// Frame-block-causal flash attention over the KV ring buffer: 8-wavefront workgroups fed by
+// LDS-DMA (gfx950, wave64, MFMA).
 //
 // Replaces the reference's make_block_mask + flex_attention pair (src/model/kv_cache.py:12-61,
 // :141-144; src/model/attn.py:116).  A key row is visible iff it is in the tail [L, L+T) or in
@@ -7,24 +8,31 @@
 // query, so the kernel builds a short list of visible slots and walks those slots of the
 // cache buffer in place, 64 keys at a time; no mask tensor and no gathered context exist.
 //
-// Work decomposition: one workgroup of 4 wavefronts per (batch, head, query tile, context
-// split).  Each wavefront owns NQB blocks of 32 queries.  Per 64-key tile:
-//   S^T[key][query] = K Q^T       v_mfma_f32_32x32x16 with A = K rows from LDS (one 16-byte
-//                                 ds_read per fragment), B = Q rows held in registers.
-//   online softmax                every lane owns ONE query column of S^T, so the row max
-//                                 and row sum are register reductions plus one
-//                                 v_permlane32_swap between the two half-waves.
-//   O^T[d][query] += V^T P^T      A = V^T fragments fetched with ds_read_b64_tr_b16 from the
-//                                 row-major V tile (the LDS transposing read of gfx950),
-//                                 B = P^T: the S^T accumulators already have the B-operand
-//                                 layout, so P never leaves registers.
-// K/V tiles go HBM -> registers -> LDS (double buffered, one barrier per tile); the global
-// loads of tile i+1 are in flight while tile i is being computed.
-// Workgroup ids are laid out so that the workgroups sharing one K/V stream (query tiles and
-// grouped query heads) run on the same XCD and hit in its L2.
+// One workgroup = 8 wavefronts = one CU (2 wavefronts per SIMD, so one wavefront's vector work
+// overlaps the other's matrix work).  Two shapes:
+//   KSPLIT = 1: 256 queries; each wavefront owns 32 queries and handles both 32-key blocks of
+//               every tile (large frames).
+//   KSPLIT = 2: 128 queries; two wavefronts share a block of 32 queries, each taking one of the
+//               two 32-key blocks of every tile, and merge their (reference, sum, O) through LDS
+//               at the end.  Twice the parallelism per query without more split-context
+//               partials (256-token frames, where the grid alone cannot fill the chip).
+// K/V tiles travel HBM -> LDS directly (global_load_lds_dwordx4, no VGPR staging) into rings
+// of 4 slots per operand, issued two to three tiles ahead.  LDS tiles are unpadded; bank
+// conflicts are avoided by XOR-swizzling 16-byte chunks, applied on the global side of the DMA
+// (lane i always lands at LDS offset 16*i) and undone in the fragment addresses.
+// Per 32-key block and wavefront:
+//   S^T = K Q^T        v_mfma_f32_32x32x16, A = K rows (ds_read_b128), B = Q in registers,
+//                      pre-multiplied by scale*log2(e); one extra MFMA (ones x -m_ref) makes the
+//                      logits leave the matrix core already shifted by the running reference.
+//   P = 2^S            v_exp_f32 + v_cvt_pk + v_dot2c row sum; each lane owns one query column.
+//   O^T += V^T P^T     A = V^T via ds_read_b64_tr_b16, B = P straight from registers.
+// The three are software-pipelined across blocks (logits of block i+1 and product of block i-1
+// run on the matrix cores while the VALU handles block i); LDS fragment reads are stated up to 15
+// reads ahead of their MFMAs, also across steps and barriers, and the order is pinned with
+// sched_barrier.  When the workgroup count leaves a partial last round of CUs, only that round's
+// (batch, kv head) units are context-split (see the planner in capi.hip).
 //
-// Roofline: 4*T*N_vis*Dh flops and 4*N_vis*Dh bytes of K/V per (batch, kv head); HBM-bound for
-// 256-query frames (with context splits to fill 256 CUs), MFMA-bound for 1024-query frames.
+// Roofline: 4*T*N_vis*Dh flops and 4*N_vis*Dh bytes of K/V per (batch, kv head).
 #include "attn_mma.h"
 #include "we_kernels.h"
 #include "../../include/we_attn.h"
@@ -32,29 +40,90 @@
 namespace we {
 
 template <int DH>
-struct AttnLds {
-  static constexpr int KSTR = DH + 8;   // K row stride: 16-byte reads of 16 consecutive rows hit all banks
-  static constexpr int VSTR = DH + 32;  // V row stride: transposing 8-byte reads of 4 rows x 64 bytes hit all banks
-  static constexpr int kBytes = 2 * BN * KSTR * 2 + 2 * BN * VSTR * 2 + (WE_MAX_SLOTS + 2) * 4;
+struct RingLds {
+  static constexpr int CPR = DH / 8;          // 16-byte chunks per row
+  static constexpr int ROW_B = DH * 2;        // bytes per K/V row
+  static constexpr int TILE_B = BN * ROW_B;   // bytes per K or V tile
+  static constexpr int SLOTS = 4;             // ring slots per operand over all wave groups
+  static constexpr int V_OFF = SLOTS * TILE_B;
+  static constexpr int MISC_OFF = 2 * SLOTS * TILE_B;
+  static constexpr int kBytes = MISC_OFF + (WE_MAX_SLOTS + 2) * 4;
 };
 
-template <typename M, int DH, int NQB>
-__global__ void __launch_bounds__(256, NQB == 1 ? 2 : 1) attn_ring_kernel(AttnParams p) {
+// chunk swizzles: physical 16-byte chunk = logical chunk ^ swz(row)
+template <int DH>
+__device__ __forceinline__ int k_swz(int row) {
+  return DH == 128 ? (row & 15) : ((row >> 1) & 7);
+}
+template <int DH>
+__device__ __forceinline__ int v_swz(int row) {
+  return DH == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2);
+}
+
+// One 1-KB LDS-DMA: lane i copies 16 bytes from gbase + voff to LDS byte lds_addr + 16*i.
+// Hidden from the compiler's counter bookkeeping on purpose; completion is awaited with
+// dma_wait<N>() (vmcnt) followed by a workgroup barrier.
+__device__ __forceinline__ void dma16(uint64_t gbase, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :
+               : "v"(voff), "s"(gbase), "s"(lds_addr)
+               : "memory");
+}
+template <int N>
+__device__ __forceinline__ void dma_wait() {
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+__device__ __forceinline__ uint64_t uniform64(uint64_t x) {
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)x);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(x >> 32));
+  return ((uint64_t)hi << 32) | lo;
+}
+
+template <int V>
+struct IntC {
+  static constexpr int value = V;
+};
+
+// ---- LDS fragment reads ---------------------------------------------------------------------
+// Left alone, the compiler keeps a single fragment read in flight ahead of the MFMA that needs
+// it, which exposes the full LDS latency on every MFMA.  The hot loop therefore states its reads
+// early in program order, several fragments ahead of their MFMAs, and pins that order with
+// sched_barrier; the reads stay ordinary loads, so the compiler still places the (counted)
+// lgkmcnt waits itself and knows the registers are in flight.
+template <int OFF>
+__device__ __forceinline__ u32x4_t lds_read128(const unsigned char* smem, uint32_t off) {
+  return *reinterpret_cast<const u32x4_t*>(smem + off + OFF);
+}
+template <int OFF>
+__device__ __forceinline__ u32x2_t lds_read_tr(const unsigned char* smem, uint32_t off) {
+  const s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(smem + off + OFF));
+  return __builtin_bit_cast(u32x2_t, v);
+}
+
+template <typename M, int DH, int KSPLIT>
+__global__ void __launch_bounds__(512, 2) attn_ring_kernel(AttnParams p) {
   typedef typename M::frag_t frag_t;
-  constexpr int KSTR = AttnLds<DH>::KSTR, VSTR = AttnLds<DH>::VSTR;
-  constexpr int KS = DH / 16;            // contraction steps of K Q^T
-  constexpr int DB = DH / 32;            // 32-row blocks of O^T
-  constexpr int BM = 128 * NQB;          // queries per workgroup
-  constexpr int CPR = DH / 8;            // 16-byte chunks per K/V row
-  constexpr int CPT = BN * CPR / 256;    // chunks per thread per tile
+  typedef RingLds<DH> L;
+  constexpr int KS = DH / 16;               // contraction steps of K Q^T
+  constexpr int DB = DH / 32;               // 32-row blocks of O^T
+  constexpr int NV = 2 * DB;                // V^T fragments of one 32-key block
+  constexpr int QW = 8 / KSPLIT;            // wavefronts with distinct query blocks
+  constexpr int BM = 32 * QW;               // queries per workgroup
+  constexpr int NST = 4;                    // ring slots per operand
+  constexpr int CPR = L::CPR, ROW_B = L::ROW_B, TILE_B = L::TILE_B;
+  constexpr int KB_B = 32 * ROW_B;          // bytes of one 32-key block of a tile
+  constexpr int RPI = 1024 / ROW_B;         // rows moved by one DMA instruction
+  constexpr int NDMA = TILE_B / 1024 / 8;   // DMA instructions per wavefront and tile operand
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  uint16_t* lds_k = reinterpret_cast<uint16_t*>(smem);  // [2][BN][KSTR]
-  uint16_t* lds_v = lds_k + 2 * BN * KSTR;              // [2][BN][VSTR]
-  int* vis = reinterpret_cast<int*>(lds_v + 2 * BN * VSTR);  // visible slots, then their count
+  int* vis = reinterpret_cast<int*>(smem + L::MISC_OFF);  // visible slots, then their count
+  const uint32_t lds0 =
+      (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, hh = lane >> 5;
+  const int qb = wave % QW;   // query block of this wavefront
+  const int hb = wave / QW;   // key block of every tile it handles when KSPLIT == 2 (else 0)
 
   // ---- which (batch, head, query tile, split) this workgroup owns; XCD = blockIdx % 8 ----
   const int xcd = blockIdx.x & 7, jj = blockIdx.x >> 3;
@@ -72,6 +141,17 @@ __global__ void __launch_bounds__(256, NQB == 1 ? 2 : 1) attn_ring_kernel(AttnPa
   const int b = unit / p.Hkv, hkv = unit - b * p.Hkv;
   const int hq_in = member / p.q_tiles, qtile = member - hq_in * p.q_tiles;
   const int h = hkv * (p.H / p.Hkv) + hq_in;
+
+  // ---- raw Q fragments: requested first so the loads overlap the slot-list construction ----
+  frag_t qf[KS];
+  const int qrow = qtile * BM + qb * 32 + l32;
+  {
+    const uint16_t* qbase = reinterpret_cast<const uint16_t*>(p.q) + b * p.qs_b + h * p.qs_h;
+    const int qr = qrow < p.T ? qrow : p.T - 1;
+    const uint16_t* src = qbase + (int64_t)qr * p.qs_t + hh * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = *reinterpret_cast<const frag_t*>(src + ks * 16);
+  }
 
   // ---- list of visible slots (the tail is pseudo-slot n_slots) ----
   if (wave == 0) {
@@ -91,68 +171,62 @@ __global__ void __launch_bounds__(256, NQB == 1 ? 2 : 1) attn_ring_kernel(AttnPa
     }
   }
   __syncthreads();
-  const int nvis = vis[WE_MAX_SLOTS + 1];
+  const int nvis = __builtin_amdgcn_readfirstlane(vis[WE_MAX_SLOTS + 1]);
+  // The list moves into registers (entry i in lane i % 64 of register i / 64) so that the hot
+  // loop can look slots up with v_readlane instead of an LDS read it would have to wait for.
+  int visr[(WE_MAX_SLOTS + 64) / 64];
+#pragma unroll
+  for (int k = 0; k < (WE_MAX_SLOTS + 64) / 64; ++k) visr[k] = (64 * k + lane < nvis) ? vis[64 * k + lane] : 0;
+  auto vis_at = [&](int i) __attribute__((always_inline)) {
+    const int l = i & 63;
+    switch (i >> 6) {
+      case 0: return __builtin_amdgcn_readlane(visr[0], l);
+      case 1: return __builtin_amdgcn_readlane(visr[1], l);
+      case 2: return __builtin_amdgcn_readlane(visr[2], l);
+      case 3: return __builtin_amdgcn_readlane(visr[3], l);
+      default: return __builtin_amdgcn_readlane(visr[4], l);
+    }
+  };
   const int tps = p.T / BN;  // tiles per slot
   const int nt = nvis * tps;
   const int t_begin = (int)((int64_t)split * nt / nsp);
   const int t_end = (int)((int64_t)(split + 1) * nt / nsp);
   const int ntile = t_end - t_begin;
 
-  // ---- Q fragments stay in registers for the whole kernel, pre-multiplied by scale*log2(e) so
-  // the matrix product yields base-2 logits directly ----
+  // ---- Q stays in registers for the whole kernel, pre-multiplied by scale*log2(e) ----
   const float c2 = p.scale_log2;
-  frag_t qf[NQB][KS];
-  int qrow[NQB];
-  {
-    const uint16_t* qbase = reinterpret_cast<const uint16_t*>(p.q) + b * p.qs_b + h * p.qs_h;
 #pragma unroll
-    for (int qb = 0; qb < NQB; ++qb) {
-      qrow[qb] = qtile * BM + wave * (32 * NQB) + qb * 32 + l32;
-      const int qr = qrow[qb] < p.T ? qrow[qb] : p.T - 1;
-      const uint16_t* src = qbase + (int64_t)qr * p.qs_t + hh * 8;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const frag_t raw = *reinterpret_cast<const frag_t*>(src + ks * 16);
-        qf[qb][ks] = M::pack8((float)raw[0] * c2, (float)raw[1] * c2, (float)raw[2] * c2, (float)raw[3] * c2,
-                              (float)raw[4] * c2, (float)raw[5] * c2, (float)raw[6] * c2, (float)raw[7] * c2);
-      }
-    }
+  for (int ks = 0; ks < KS; ++ks) {
+    const frag_t raw = qf[ks];
+    qf[ks] = M::pack8((float)raw[0] * c2, (float)raw[1] * c2, (float)raw[2] * c2, (float)raw[3] * c2,
+                      (float)raw[4] * c2, (float)raw[5] * c2, (float)raw[6] * c2, (float)raw[7] * c2);
   }
 
   const int64_t cap = p.L + p.T;
-  const uint16_t* kbase =
-      reinterpret_cast<const uint16_t*>(p.kv) + ((int64_t)b * p.Hkv + hkv) * cap * DH;
-  const uint16_t* vbase = kbase + (int64_t)p.B * p.Hkv * cap * DH;
+  const uint64_t kbase = (uint64_t)(uintptr_t)p.kv + (uint64_t)(((int64_t)b * p.Hkv + hkv) * cap) * ROW_B;
+  const uint64_t vbase = kbase + (uint64_t)((int64_t)p.B * p.Hkv * cap) * ROW_B;
 
-  // ---- software pipeline -------------------------------------------------------------------
-  // Iteration `it` holds the logits of tile `it` (s_cur), computes the logits of tile it+1 and
-  // the P*V product of tile it-1 on the matrix cores while the VALU turns s_cur into
-  // probabilities.  LDS: K(it+1) in kb[(it+1)&1], V(it-1) in vb[(it-1)&1]; the stores of K(it+2)
-  // and V(it) go into the two buffers nobody reads during this iteration, so one barrier per
-  // tile is enough.  Global loads run one iteration ahead of their LDS store (K(it+3), V(it+1)).
-  // Tile indices past the end are clamped (the last tile is re-loaded and its logits recomputed
-  // once), which keeps the loop body free of branches.
-  //
-  // The logits leave the matrix cores already shifted by the running reference m_ref: one extra
-  // MFMA per 32-key block multiplies a column of ones (K side) with a fragment holding -m_ref
-  // (Q side; m_ref is kept representable in the element type so the shift is exact).  The VALU
-  // work per element is then exp2, a pack, and half a dot2 for the row sum.  m_ref is raised
-  // only when a row sum shows a probability above 2^8 (then that tile is redone exactly); being
-  // larger than the true running max is never needed for fp32 accumulators.
-  u32x4_t kreg[CPT], vreg[CPT];
-  const int ld_r = tid / CPR, ld_c8 = tid % CPR;  // chunk c = tid + 256*i -> row ld_r + i*(256/CPR)
-  struct TileWalk {  // position of a load stream in this split's list of visible tiles
+  // ---- DMA plumbing ----
+  // Instruction i of this wavefront moves rows [q*RPI, (q+1)*RPI) of a tile, q = wave + 8*i.
+  uint32_t kvoff[NDMA], vvoff[NDMA];
+#pragma unroll
+  for (int i = 0; i < NDMA; ++i) {
+    const int row = (wave + i * 8) * RPI + lane / CPR;
+    const int phys = lane % CPR;
+    kvoff[i] = row * ROW_B + ((phys ^ k_swz<DH>(row)) << 4);
+    vvoff[i] = row * ROW_B + ((phys ^ v_swz<DH>(row)) << 4);
+  }
+  struct TileWalk {  // position of a load stream in the split's list of visible tiles
     int sidx, sub, left;
   };
-  auto walk_init = [&](int ti) __attribute__((always_inline)) {
+  auto walk_init = [&]() __attribute__((always_inline)) {
     TileWalk w;
-    const int g = t_begin + (ti < ntile ? ti : ntile - 1);
-    w.sidx = g / tps;
-    w.sub = g - w.sidx * tps;
-    w.left = ntile - 1 - (ti < ntile ? ti : ntile - 1);
+    w.sidx = t_begin / tps;
+    w.sub = t_begin - w.sidx * tps;
+    w.left = ntile - 1;
     return w;
   };
-  auto walk_next = [&](TileWalk& w) __attribute__((always_inline)) {
+  auto walk_next = [&](TileWalk& w) __attribute__((always_inline)) {  // stays on the last tile
     if (w.left > 0) {
       --w.left;
       if (++w.sub == tps) {
@@ -161,367 +235,428 @@ __global__ void __launch_bounds__(256, NQB == 1 ? 2 : 1) attn_ring_kernel(AttnPa
       }
     }
   };
-  auto tile_ptr = [&](const uint16_t* base, const TileWalk& w) __attribute__((always_inline)) {
-    const int slot = __builtin_amdgcn_readfirstlane(vis[w.sidx]);
-    const int64_t row0 = (int64_t)slot * p.T + (int64_t)w.sub * BN;
-    return base + (row0 + ld_r) * DH + ld_c8 * 8;
+  // byte offset of a tile inside its (batch, kv head) plane; fits 32 bits (checked on the host)
+  auto tile_off = [&](const TileWalk& w) __attribute__((always_inline)) {
+    return (uint32_t)(vis_at(w.sidx) * p.T + w.sub * BN) * (uint32_t)ROW_B;
   };
-  auto gload = [&](u32x4_t(&r)[CPT], const uint16_t* src) __attribute__((always_inline)) {
+  const uint64_t kplane = uniform64(kbase), vplane = uniform64(vbase);
+  auto dma_k = [&](uint32_t off, int slot) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < CPT; ++i)
-      r[i] = *reinterpret_cast<const u32x4_t*>(src + (int64_t)i * (256 / CPR) * DH);
+    for (int i = 0; i < NDMA; ++i)
+      dma16(kplane, kvoff[i] + off, __builtin_amdgcn_readfirstlane(lds0 + slot * TILE_B + (wave + i * 8) * 1024));
   };
-  auto lstore = [&](uint16_t* dst, int stride, const u32x4_t(&r)[CPT]) __attribute__((always_inline)) {
+  auto dma_v = [&](uint32_t off, int slot) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < CPT; ++i) *reinterpret_cast<u32x4_t*>(dst + i * (256 / CPR) * stride) = r[i];
+    for (int i = 0; i < NDMA; ++i)
+      dma16(vplane, vvoff[i] + off,
+            __builtin_amdgcn_readfirstlane(lds0 + L::V_OFF + slot * TILE_B + (wave + i * 8) * 1024));
   };
-  uint16_t* const k_st = lds_k + ld_r * KSTR + ld_c8 * 8;  // this thread's staging slots
-  uint16_t* const v_st = lds_v + ld_r * VSTR + ld_c8 * 8;
-  // per-lane offsets of the fragment reads
-  const uint16_t* const k_rd = lds_k + l32 * KSTR + hh * 8;
-  const uint16_t* const v_rd =
-      lds_v + (4 * hh + ((lane & 15) >> 2)) * VSTR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
-  f32x16_t o[NQB][DB];
-  float m_ref[NQB], l_run[NQB];
-#pragma unroll
-  for (int qb = 0; qb < NQB; ++qb) {
-    m_ref[qb] = -INFINITY;
-    l_run[qb] = 0.f;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) o[qb][db][i] = 0.f;
+  // ---- fragment read addresses (byte offsets into smem) ----
+  // K row l32 of a key block, logical chunk 2*ks + hh: physical chunk bits [3:1] are
+  // ks ^ (swz >> 1), so the address for step ks is the step-0 address with bits 5.. flipped.
+  uint32_t k_rd;
+  {
+    const int x = k_swz<DH>(l32);
+    k_rd = hb * KB_B + l32 * ROW_B + ((((x >> 1) << 1) | (hh ^ (x & 1))) << 4);
+  }
+  // V rows 4*hh + r (r = lane bits 3:2) of each 8-row group, logical chunk 4*db + c.
+  uint32_t v_rd;
+  {
+    const int r = 4 * hh + ((lane & 15) >> 2);
+    const int y = v_swz<DH>(r) >> 2;
+    const int c = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
+    v_rd = L::V_OFF + hb * KB_B + r * ROW_B + ((y * 4 + c) << 4) + (lane & 1) * 8;
   }
 
+  f32x16_t o[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
+  float m_ref = -INFINITY, l_run = 0.f;
+
   const f32x16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  const float kDead = 3.0e4f;  // shift of logits that must not count (tiles past the end)
   // K-side fragment of the shift product: contraction index 0 is one for every key
   frag_t ones_frag = __builtin_bit_cast(frag_t, u32x4_t{0u, 0u, 0u, 0u});
   if (hh == 0) ones_frag[0] = (typename M::elem_t)1.0f;
-  // Q-side fragment: contraction index 0 carries -m_ref of this lane's query
-  frag_t shift[NQB];
-  auto set_shift = [&](int qb) __attribute__((always_inline)) {
-    shift[qb] = __builtin_bit_cast(frag_t, u32x4_t{0u, 0u, 0u, 0u});
-    if (hh == 0) shift[qb][0] = (typename M::elem_t)(-m_ref[qb]);
+  // Q-side fragments: contraction index 0 carries -m_ref of this lane's query, or -kDead
+  frag_t shift = __builtin_bit_cast(frag_t, u32x4_t{0u, 0u, 0u, 0u});
+  frag_t dead = shift;
+  if (hh == 0) dead[0] = (typename M::elem_t)(-kDead);
+  auto set_shift = [&]() __attribute__((always_inline)) {
+    shift = __builtin_bit_cast(frag_t, u32x4_t{0u, 0u, 0u, 0u});
+    if (hh == 0) shift[0] = (typename M::elem_t)(-m_ref);
   };
 
-  // logits of one 64-key tile in LDS buffer `kt`, already minus m_ref when `shifted`
-  auto logits = [&](f32x16_t(&s)[NQB][2], const uint16_t* kt, bool shifted) __attribute__((always_inline)) {
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-      for (int qb = 0; qb < NQB; ++qb)
-        s[qb][kb] = shifted ? M::mma(ones_frag, shift[qb], zero16) : zero16;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const frag_t a = *reinterpret_cast<const frag_t*>(kt + kb * 32 * KSTR + ks * 16);
-#pragma unroll
-        for (int qb = 0; qb < NQB; ++qb) s[qb][kb] = M::mma(a, qf[qb][ks], s[qb][kb]);
-      }
-    }
-  };
-  // O^T += V^T P^T for one 64-key tile in LDS buffer `vt`
-  auto accumulate = [&](const frag_t(&pf)[NQB][4], const uint16_t* vt) __attribute__((always_inline)) {
-#pragma unroll
-    for (int m = 0; m < 4; ++m) {
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        const uint16_t* va = vt + 16 * m * VSTR + 32 * db;
-        const s16x4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(va));
-        const s16x4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(va + 8 * VSTR));
-        typedef short s16x8_t __attribute__((ext_vector_type(8)));
-        const s16x8_t a8 = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
-        const frag_t a = __builtin_bit_cast(frag_t, a8);
-#pragma unroll
-        for (int qb = 0; qb < NQB; ++qb) o[qb][db] = M::mma(a, pf[qb][m], o[qb][db]);
-      }
-    }
-  };
-  // probabilities of one tile from its shifted logits: p = 2^s, packed to the element type;
-  // returns this half-wave's share of the row sum (of the rounded values)
-  auto probabilities = [&](frag_t(&pf)[4], const f32x16_t(&s)[2], float sub) __attribute__((always_inline)) {
+  // probabilities of one 32-key block from its shifted logits: p = 2^(s - sub), packed to the
+  // element type; returns this half-wave's share of the row sum (of the rounded values)
+  auto probabilities = [&](frag_t(&pf)[2], const f32x16_t& s, float sub) __attribute__((always_inline)) {
     float rs = 0.f;
 #pragma unroll
-    for (int m = 0; m < 4; ++m) {
-      const f32x16_t& sv = s[m >> 1];
-      const int r0 = 8 * (m & 1);
+    for (int m = 0; m < 2; ++m) {
       float e[8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) e[j] = __builtin_amdgcn_exp2f(sv[r0 + j] - sub);
+      for (int j = 0; j < 8; ++j) e[j] = __builtin_amdgcn_exp2f(s[8 * m + j] - sub);
       pf[m] = M::pack8(e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7]);
 #pragma unroll
       for (int j = 0; j < 4; ++j) rs = M::add_pair(rs, pf[m], j);
     }
     return rs;
   };
-  auto tile_max = [&](const f32x16_t(&s)[2]) __attribute__((always_inline)) {
-    float mx = s[0][0];
+  auto block_max = [&](const f32x16_t& s) __attribute__((always_inline)) {
+    float mx = s[0];
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kb][i]);
+    for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s[i]);
     float lo, up;
     half_wave_pair(mx, lo, up);
     return fmaxf(lo, up);
   };
 
-  if (ntile > 0) {
-    frag_t p_prev[NQB][4];
-    f32x16_t s_cur[NQB][2];
-    {
-      // zero V buffer 1 and P so that the first iteration's product adds exact zeros
-      const u32x4_t z = {0u, 0u, 0u, 0u};
-      for (int i = tid; i < BN * VSTR / 8; i += 256)
-        *reinterpret_cast<u32x4_t*>(lds_v + BN * VSTR + i * 8) = z;
-#pragma unroll
-      for (int qb = 0; qb < NQB; ++qb)
-#pragma unroll
-        for (int m = 0; m < 4; ++m) p_prev[qb][m] = __builtin_bit_cast(frag_t, z);
+  // The pipeline runs on 32-key blocks.  One step computes, for this wavefront,
+  //   matrix cores: the shifted logits of the block read at K offset KOFF (-> s_next) and the
+  //                 product of the previous block's probabilities with the V block at VOFF;
+  //   VALU:         the probabilities of the current block (s_cur -> p_cur).
+  // LDS reads are issued in consumption order - K fragments 0..KS-1, then the NV V^T fragments
+  // (two transposing reads each) - running up to 15 reads ahead of the MFMAs.
+  bool pending = false;   // an accumulator rescale decided in the previous step is due
+  float alpha = 1.f;
+  frag_t p_prev[2];
+  f32x16_t s_cur;
+  // Fragment registers live across steps: every step starts with its first PRE reads (all K
+  // fragments and the first V^T fragment) already in flight, issued during the previous step.
+  constexpr int PRE = KS + 2;
+  u32x4_t kf[KS];
+  u32x2_t v0[NV], v1[NV];
+  auto read_k = [&](auto koff_c, int ks) __attribute__((always_inline)) {
+    kf[ks] = lds_read128<decltype(koff_c)::value>(smem, k_rd ^ (ks << 5));
+  };
+  auto read_v = [&](auto voff_c, int i) __attribute__((always_inline)) {  // fragment i = (m, db) = (i / DB, i % DB)
+    constexpr int VOFF = decltype(voff_c)::value;
+    const uint32_t a = v_rd ^ ((i % DB) << 6);
+    if (i / DB == 0) {
+      v0[i] = lds_read_tr<VOFF>(smem, a);
+      v1[i] = lds_read_tr<VOFF + 8 * ROW_B>(smem, a);
+    } else {
+      v0[i] = lds_read_tr<VOFF + 16 * ROW_B>(smem, a);
+      v1[i] = lds_read_tr<VOFF + 24 * ROW_B>(smem, a);
     }
-    TileWalk kw = walk_init(0), vw = walk_init(0);
-    gload(kreg, tile_ptr(kbase, kw));  // K(0)
-    walk_next(kw);
-    gload(vreg, tile_ptr(kbase, kw));  // K(1)
-    walk_next(kw);
-    lstore(k_st, KSTR, kreg);
-    lstore(k_st + BN * KSTR, KSTR, vreg);
-    gload(kreg, tile_ptr(kbase, kw));  // K(2)
-    walk_next(kw);
-    gload(vreg, tile_ptr(vbase, vw));  // V(0)
-    walk_next(vw);
-    __syncthreads();
-    // first tile: plain logits, reference = its row max, then shift by hand
-    logits(s_cur, k_rd, false);
+  };
+  auto prefetch = [&](auto koff_c, auto voff_c) __attribute__((always_inline)) {
 #pragma unroll
-    for (int qb = 0; qb < NQB; ++qb) {
-      m_ref[qb] = M::round_up(tile_max(s_cur[qb]));
-      set_shift(qb);
+    for (int ks = 0; ks < KS; ++ks) read_k(koff_c, ks);
+    read_v(voff_c, 0);
+  };
+  auto step = [&](auto koff_c, auto voff_c, auto nkoff_c, auto nvoff_c, bool live, auto&& mid) __attribute__((always_inline)) {
+    if (pending) {
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
+      for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) s_cur[qb][kb][i] -= m_ref[qb];
+        for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
     }
-    __syncthreads();  // K buffer 0 is overwritten by the first iteration
+    pending = false;
 
-    // A raise decided in iteration it rescales the accumulators after the product of tile it-1
-    // and before that of tile it, i.e. at the top of iteration it+1; with the branch there the
-    // rest of the body stays one basic block for the scheduler to interleave.
-    bool pending = false;
-    float alpha[NQB];
-#pragma unroll
-    for (int qb = 0; qb < NQB; ++qb) alpha[qb] = 1.f;
-    auto rescale = [&]() __attribute__((always_inline)) {
-#pragma unroll
-      for (int qb = 0; qb < NQB; ++qb)
-#pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) o[qb][db][i] *= alpha[qb];
+    // reads issued since this step's read 0 / next own V fragment / next-step read pairs issued
+    int issued = PRE, vnext = 1, npair = 0;
+    constexpr int NPAIR = PRE / 2;            // the next step's first reads go out two at a time
+    constexpr int I0 = NV - 1 - NPAIR;        // ... after the product MFMAs I0, I0+1, ...
+    auto next_pair = [&]() __attribute__((always_inline)) {
+      if (2 * npair < KS) {
+        read_k(nkoff_c, 2 * npair);
+        read_k(nkoff_c, 2 * npair + 1);
+      } else {
+        read_v(nvoff_c, 0);
+      }
+      ++npair;
+      issued += 2;
     };
 
-    for (int it = 0; it < ntile; ++it) {
-      if (pending) rescale();
-      pending = false;
-      const int cur = it & 1, nxt = cur ^ 1;
-      lstore(k_st + cur * BN * KSTR, KSTR, kreg);  // K(it+2)
-      lstore(v_st + cur * BN * VSTR, VSTR, vreg);  // V(it)
-      gload(kreg, tile_ptr(kbase, kw));            // K(it+3)
-      walk_next(kw);
-      gload(vreg, tile_ptr(vbase, vw));            // V(it+1)
-      walk_next(vw);
-
-      // matrix cores: shifted logits of tile it+1
-      f32x16_t s_next[NQB][2];
-      logits(s_next, k_rd + nxt * BN * KSTR, true);
-
-      // VALU: probabilities of tile it
-      frag_t p_cur[NQB][4];
-      float rs[NQB];
-      bool bad = false;
+    // From here to the end of the product the issue order is pinned statement by statement
+    // (sched_barrier): MFMA, the reads that refill the queue, a slice of the VALU work.
+    __builtin_amdgcn_sched_barrier(0);
+    f32x16_t s_next = M::mma(ones_frag, live ? shift : dead, zero16);
+    frag_t p_cur[2];
+    float e[16];
+    float rs = 0.f;
 #pragma unroll
-      for (int qb = 0; qb < NQB; ++qb) {
-        rs[qb] = probabilities(p_cur[qb], s_cur[qb], 0.f);
-        bad = bad || !(rs[qb] <= 256.f);
+    for (int ks = 0; ks < KS; ++ks) {
+      s_next = M::mma(__builtin_bit_cast(frag_t, kf[ks]), qf[ks], s_next);
+      // keep the read queue full without exceeding the 15 reads the counter can track
+      if (vnext < NV && ks <= 12 - KS) {
+        read_v(voff_c, vnext);
+        ++vnext;
+        issued += 2;
       }
-
-      // matrix cores: O += P(it-1) V(it-1)
-      accumulate(p_prev, v_rd + nxt * BN * VSTR);
-
-      if (__ballot(bad) != 0ull) {
-        // Rare: some probability of this tile may exceed 2^8.  Raise the reference of the rows
-        // that need it, redo the tile's probabilities exactly, and re-base the logits of the
-        // next tile, which were produced with the old reference.
+      // VALU slice: 16 / KS exponentials of the current block
 #pragma unroll
-        for (int qb = 0; qb < NQB; ++qb) {
-          const float mx = tile_max(s_cur[qb]);
-          const float m_new = mx > 0.f ? M::round_up(m_ref[qb] + mx) : m_ref[qb];
-          const float delta = m_new - m_ref[qb];
-          alpha[qb] = __builtin_amdgcn_exp2f(-delta);
-          rs[qb] = probabilities(p_cur[qb], s_cur[qb], delta);
-          l_run[qb] *= alpha[qb];
-          m_ref[qb] = m_new;
-          set_shift(qb);
-#pragma unroll
-          for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) s_next[qb][kb][i] -= delta;
-        }
-        pending = true;
-      }
-#pragma unroll
-      for (int qb = 0; qb < NQB; ++qb) {
-        l_run[qb] += rs[qb];
-#pragma unroll
-        for (int m = 0; m < 4; ++m) p_prev[qb][m] = p_cur[qb][m];
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb) s_cur[qb][kb] = s_next[qb][kb];
-      }
-      __syncthreads();
+      for (int t = 0; t < 16 / KS; ++t)
+        e[ks * (16 / KS) + t] = __builtin_amdgcn_exp2f(s_cur[ks * (16 / KS) + t]);
+      __builtin_amdgcn_sched_barrier(0);
     }
-    if (pending) rescale();
-    accumulate(p_prev, v_rd + ((ntile - 1) & 1) * BN * VSTR);
-  }
-  float m_run[NQB];
+    mid();  // the tile DMAs of this iteration go out here, under the MFMAs already queued
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-  for (int qb = 0; qb < NQB; ++qb) m_run[qb] = m_ref[qb];
+    for (int i = 0; i < NV; ++i) {
+      if (vnext < NV) {  // reads 0..KS+2i-1 have completed: room for one more fragment
+        read_v(voff_c, vnext);
+        ++vnext;
+        issued += 2;
+      }
+      typedef unsigned int u32x4v __attribute__((ext_vector_type(4)));
+      const u32x4v a4 = __builtin_shufflevector(v0[i], v1[i], 0, 1, 2, 3);
+      o[i % DB] = M::mma(__builtin_bit_cast(frag_t, a4), p_prev[i / DB], o[i % DB]);
+      if (i >= I0 && npair < NPAIR) next_pair();
+      // VALU slices: pack the two 16-key halves, then their row sums
+      if (i == 0) p_cur[0] = M::pack8(e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7]);
+      if (i == 1) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) rs = M::add_pair(rs, p_cur[0], t);
+      }
+      if (i == 2) p_cur[1] = M::pack8(e[8], e[9], e[10], e[11], e[12], e[13], e[14], e[15]);
+      if (i == 3) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) rs = M::add_pair(rs, p_cur[1], t);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+
+    if (__ballot(!(rs <= 256.f)) != 0ull) {
+      // Rare: some probability of this block may exceed 2^8.  Raise the reference of the rows
+      // that need it, redo the block's probabilities exactly, and re-base the logits of the next
+      // block, which were produced with the old reference.
+      const float mx = block_max(s_cur);
+      const float m_new = mx > 0.f ? M::round_up(m_ref + mx) : m_ref;
+      const float delta = m_new - m_ref;
+      alpha = __builtin_amdgcn_exp2f(-delta);
+      rs = probabilities(p_cur, s_cur, delta);
+      l_run *= alpha;
+      m_ref = m_new;
+      set_shift();
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s_next[i] -= delta;
+      pending = true;
+    }
+    l_run += rs;
+    p_prev[0] = p_cur[0];
+    p_prev[1] = p_cur[1];
+    s_cur = s_next;
+  };
+
+  if (ntile > 0) {
+    {
+      // zero V slot 3, which stands in for "tile -1", and P, so the first product adds zeros
+      const u32x4_t z = {0u, 0u, 0u, 0u};
+      unsigned char* vz = smem + L::V_OFF + 3 * TILE_B;
+      for (int i = tid; i < TILE_B / 16; i += 512) *reinterpret_cast<u32x4_t*>(vz + i * 16) = z;
+      p_prev[0] = __builtin_bit_cast(frag_t, z);
+      p_prev[1] = __builtin_bit_cast(frag_t, z);
+    }
+    // Iteration j issues K(j+KA) and V(j+2) (KA = 3, or 4 when every wavefront handles one key
+    // block per tile and prefetches its next fragments across the barrier); the prologue issues
+    // what the iterations before 0 would have.
+    constexpr int KA = KSPLIT == 1 ? 3 : 4;
+    // The V stream trails the K stream by KA - 2 tiles, so it reuses the K stream's offsets.
+    TileWalk kw = walk_init();
+    uint32_t off1, off2;  // offsets of the last and the last-but-one tile the K stream visited
+    {
+      const uint32_t o0 = tile_off(kw); walk_next(kw);
+      const uint32_t o1 = tile_off(kw); walk_next(kw);
+      const uint32_t o2 = tile_off(kw); walk_next(kw);
+      dma_k(o0, 0);
+      dma_k(o1, 1);
+      if (KSPLIT == 2) dma_k(o2, 2);
+      dma_v(o0, 0);
+      if (KSPLIT == 1) {
+        dma_k(o2, 2);
+        off1 = o2; off2 = o1;
+      } else {
+        const uint32_t o3 = tile_off(kw); walk_next(kw);
+        dma_k(o3, 3);
+        off1 = o3; off2 = o2;
+      }
+      dma_v(o1, 1);
+    }
+    dma_wait<(KA + 1) * NDMA>();
+    __syncthreads();  // K(0) and the zeroed V slot are in LDS
+    // first block: plain logits, reference = its row max, shifted by hand
+    {
+      s_cur = zero16;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const frag_t a = *reinterpret_cast<const frag_t*>(smem + (k_rd ^ (ks << 5)));
+        s_cur = M::mma(a, qf[ks], s_cur);
+      }
+      m_ref = M::round_up(block_max(s_cur));
+      set_shift();
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s_cur[i] -= m_ref;
+    }
+    dma_wait<2 * NDMA>();
+    __syncthreads();  // everything but the last K and V tile issued so far has landed
+    // first reads of the first step
+    if (KSPLIT == 1) prefetch(IntC<KB_B>(), IntC<3 * TILE_B + KB_B>());
+    else prefetch(IntC<TILE_B>(), IntC<3 * TILE_B>());
+
+    // one tile iteration with compile-time ring positions (JM = j mod 4)
+    auto iteration = [&](int j, auto jm_c) __attribute__((always_inline)) {
+      constexpr int JM = decltype(jm_c)::value;
+      auto issue_dma = [&]() __attribute__((always_inline)) {
+        const uint32_t o = tile_off(kw);
+        walk_next(kw);
+        dma_k(o, (JM + KA) % NST);                       // K(j+KA)
+        dma_v(KA == 3 ? off1 : off2, (JM + 2) % NST);    // V(j+2)
+        off2 = off1;
+        off1 = o;
+      };
+      auto nothing = [&]() __attribute__((always_inline)) {};
+      if (KSPLIT == 1) {
+        // block (j, 0) -> probabilities; logits of (j, 1); product of (j-1, 1)
+        step(IntC<JM * TILE_B + KB_B>(), IntC<((JM + 3) % NST) * TILE_B + KB_B>(),
+             IntC<((JM + 1) % NST) * TILE_B>(), IntC<JM * TILE_B>(), true, issue_dma);
+        // block (j, 1) -> probabilities; logits of (j+1, 0); product of (j, 0)
+        step(IntC<((JM + 1) % NST) * TILE_B>(), IntC<JM * TILE_B>(),
+             IntC<((JM + 1) % NST) * TILE_B + KB_B>(), IntC<JM * TILE_B + KB_B>(), j + 1 < ntile, nothing);
+      } else {
+        // block (j, hb) -> probabilities; logits of (j+1, hb); product of (j-1, hb)
+        step(IntC<((JM + 1) % NST) * TILE_B>(), IntC<((JM + 3) % NST) * TILE_B>(),
+             IntC<((JM + 2) % NST) * TILE_B>(), IntC<JM * TILE_B>(), j + 1 < ntile, issue_dma);
+      }
+      dma_wait<2 * NDMA>();  // all but this iteration's two tiles have landed (this wavefront's part)
+      __syncthreads();
+    };
+
+    int j = 0;
+    for (; j + 4 <= ntile; j += 4) {
+      iteration(j, IntC<0>());
+      iteration(j + 1, IntC<1>());
+      iteration(j + 2, IntC<2>());
+      iteration(j + 3, IntC<3>());
+    }
+    if (j < ntile) { iteration(j, IntC<0>()); ++j; }
+    if (j < ntile) { iteration(j, IntC<1>()); ++j; }
+    if (j < ntile) { iteration(j, IntC<2>()); ++j; }
+
+    // product of the last block: (ntile-1, 1) for full-tile wavefronts, (ntile-1, hb) otherwise
+    if (pending) {
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+    }
+    {
+      const int last = (ntile - 1) % NST;
+      const unsigned char* vt = smem + v_rd + last * TILE_B + (KSPLIT == 1 ? KB_B : 0);
+#pragma unroll
+      for (int m = 0; m < 2; ++m) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const unsigned char* va = smem + ((uint32_t)(vt - smem) ^ (db << 6)) + 16 * m * ROW_B;
+          const s16x4_t a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(va));
+          const s16x4_t a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(va + 8 * ROW_B));
+          typedef short s16x8_t __attribute__((ext_vector_type(8)));
+          const s16x8_t a8 = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
+          o[db] = M::mma(__builtin_bit_cast(frag_t, a8), p_prev[m], o[db]);
+        }
+      }
+    }
+    dma_wait<0>();  // no DMA may still be writing LDS when the rings are reused or the CU is freed
+  }
+
+  float lo, up;
+  half_wave_pair(l_run, lo, up);
+  float l_tot = lo + up;
+
+  if (KSPLIT == 2) {
+    // ---- the two wavefronts of a query block merge their (m, l, O) through LDS ----
+    __syncthreads();  // every wavefront is done with the rings
+    float* mb = reinterpret_cast<float*>(smem) + (qb * (DB * 16 + 2)) * 64 + lane;
+    if (hb == 1) {
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) mb[(db * 16 + i) * 64] = o[db][i];
+      mb[(DB * 16) * 64] = m_ref;
+      mb[(DB * 16 + 1) * 64] = l_tot;
+    }
+    __syncthreads();
+    if (hb == 1) return;
+    const float m1 = mb[(DB * 16) * 64], l1 = mb[(DB * 16 + 1) * 64];
+    const float mm = fmaxf(m_ref, m1);
+    if (mm > -INFINITY) {
+      const float a0 = __builtin_amdgcn_exp2f(m_ref - mm), a1 = __builtin_amdgcn_exp2f(m1 - mm);
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[db][i] = a0 * o[db][i] + a1 * mb[(db * 16 + i) * 64];
+      l_tot = a0 * l_tot + a1 * l1;
+      m_ref = mm;
+    }
+  }
 
   // ---- epilogue ----
   const int64_t rows = (int64_t)p.B * p.H * p.T - p.ws_row0;  // rows in the workspace
+  const bool valid = qrow < p.T;
+  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  const int64_t row = ((int64_t)b * p.H + h) * p.T + qrow;
+  if (nsp > 1 && valid && hh == 0) {
+    float2 ml = make_float2(m_ref, l_tot);
+    *reinterpret_cast<float2*>(p.ws_ml + ((int64_t)split * rows + (row - p.ws_row0)) * 2) = ml;
+  }
 #pragma unroll
-  for (int qb = 0; qb < NQB; ++qb) {
-    float lo, up;
-    half_wave_pair(l_run[qb], lo, up);
-    const float l_tot = lo + up;
-    const bool valid = qrow[qb] < p.T;
-    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-    const int64_t row = ((int64_t)b * p.H + h) * p.T + qrow[qb];
-    if (nsp > 1 && valid && hh == 0) {
-      float2 ml = make_float2(m_run[qb], l_tot);
-      *reinterpret_cast<float2*>(p.ws_ml + ((int64_t)split * rows + (row - p.ws_row0)) * 2) = ml;
-    }
+  for (int db = 0; db < DB; ++db) {
 #pragma unroll
-    for (int db = 0; db < DB; ++db) {
+    for (int c = 0; c < 4; c += 2) {
+      // register quad c holds head-dim rows 8c + 4*half + 0..3; after the swap a lane of the
+      // lower half owns rows 8c..8c+7 and a lane of the upper half rows 8(c+1)..8(c+1)+7.
+      float f[8];
 #pragma unroll
-      for (int c = 0; c < 4; c += 2) {
-        // register quad c holds head-dim rows 8c + 4*half + 0..3; after the swap a lane of the
-        // lower half owns rows 8c..8c+7 and a lane of the upper half rows 8(c+1)..8(c+1)+7.
-        float f[8];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(o[qb][db][4 * c + e] * inv),
-                                                    __float_as_uint(o[qb][db][4 * c + 4 + e] * inv),
-                                                    false, false);
-          f[e] = __uint_as_float(r[0]);
-          f[4 + e] = __uint_as_float(r[1]);
-        }
-        const int d0 = 32 * db + 8 * (c + hh);
-        if (valid) {
-          if (nsp == 1) {
-            uint16_t* dst = reinterpret_cast<uint16_t*>(p.out) + b * p.os_b + h * p.os_h +
-                            (int64_t)qrow[qb] * p.os_t + d0;
-            *reinterpret_cast<frag_t*>(dst) = M::pack8(f[0], f[1], f[2], f[3], f[4], f[5], f[6], f[7]);
-          } else {
-            uint16_t* dst = p.ws_o + ((int64_t)split * rows + (row - p.ws_row0)) * DH + d0;
-            *reinterpret_cast<frag_t*>(dst) = M::pack8(f[0], f[1], f[2], f[3], f[4], f[5], f[6], f[7]);
-          }
+      for (int e = 0; e < 4; ++e) {
+        auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(o[db][4 * c + e] * inv),
+                                                  __float_as_uint(o[db][4 * c + 4 + e] * inv), false, false);
+        f[e] = __uint_as_float(r[0]);
+        f[4 + e] = __uint_as_float(r[1]);
+      }
+      const int d0 = 32 * db + 8 * (c + hh);
+      if (valid) {
+        if (nsp == 1) {
+          uint16_t* dst = reinterpret_cast<uint16_t*>(p.out) + b * p.os_b + h * p.os_h +
+                          (int64_t)qrow * p.os_t + d0;
+          *reinterpret_cast<frag_t*>(dst) = M::pack8(f[0], f[1], f[2], f[3], f[4], f[5], f[6], f[7]);
+        } else {
+          uint16_t* dst = p.ws_o + ((int64_t)split * rows + (row - p.ws_row0)) * DH + d0;
+          *reinterpret_cast<frag_t*>(dst) = M::pack8(f[0], f[1], f[2], f[3], f[4], f[5], f[6], f[7]);
         }
       }
     }
   }
 }
 
-// Second pass of the split-context path.  Every split left, per query row, its normalised
-// output O_s (element type), its reference m_s (log2 domain) and its sum l_s; the result is
-// sum_s w_s O_s / sum_s w_s with w_s = 2^(m_s - max m) * l_s.  One thread per (row, 8 columns).
-template <typename M, int DH>
-__global__ void __launch_bounds__(256) attn_combine_kernel(AttnParams p) {
-  typedef typename M::frag_t frag_t;
-  const int64_t rows = (int64_t)p.B * p.H * p.T - p.ws_row0;  // rows that were split
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= rows * (DH / 8)) return;
-  const int64_t row = idx / (DH / 8);  // workspace row; query row = row + ws_row0
-  const int dg = (int)(idx % (DH / 8));
-  // Splits are merged eight at a time with all sixteen loads of a batch issued before the first
-  // use (a plain loop over a run-time split count would serialise one memory round trip per split).
-  float mmax = -INFINITY, den = 0.f;
-  float acc[8];
-#pragma unroll
-  for (int j = 0; j < 8; ++j) acc[j] = 0.f;
-  for (int s0 = 0; s0 < p.n_splits; s0 += 8) {
-    float2 ml[8];
-    frag_t ov[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int s = s0 + j < p.n_splits ? s0 + j : p.n_splits - 1;  // clamp: duplicates get weight 0 below
-      ml[j] = *reinterpret_cast<const float2*>(p.ws_ml + ((int64_t)s * rows + row) * 2);
-      ov[j] = *reinterpret_cast<const frag_t*>(p.ws_o + ((int64_t)s * rows + row) * DH + dg * 8);
-    }
-    float bmax = mmax;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) bmax = fmaxf(bmax, ml[j].x);
-    const float carry = bmax > -INFINITY ? __builtin_amdgcn_exp2f(mmax - bmax) : 0.f;  // 0 on the first batch
-    den *= carry;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) acc[j] *= carry;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const float w = (s0 + j < p.n_splits && ml[j].y > 0.f) ? __builtin_amdgcn_exp2f(ml[j].x - bmax) * ml[j].y : 0.f;
-      den += w;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] += w * (float)ov[j][e];
-    }
-    mmax = bmax;
-  }
-  const float inv = 1.f / den;
-  const int64_t qrow = row + p.ws_row0;
-  const int t = (int)(qrow % p.T);
-  const int64_t bh = qrow / p.T;
-  const int h = (int)(bh % p.H);
-  const int b = (int)(bh / p.H);
-  uint16_t* dst = reinterpret_cast<uint16_t*>(p.out) + b * p.os_b + h * p.os_h + (int64_t)t * p.os_t + dg * 8;
-  *reinterpret_cast<frag_t*>(dst) = M::pack8(acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv, acc[4] * inv,
-                                             acc[5] * inv, acc[6] * inv, acc[7] * inv);
-}
-
-template <typename M, int DH, int NQB>
-static hipError_t launch_attn_t(const AttnParams& p, hipStream_t stream) {
+template <typename M, int DH, int KSPLIT>
+static hipError_t launch_ring_t(const AttnParams& p, hipStream_t stream) {
   static bool configured = false;
-  const int lds = AttnLds<DH>::kBytes;
+  const int lds = RingLds<DH>::kBytes;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_ring_kernel<M, DH, NQB>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_ring_kernel<M, DH, KSPLIT>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
     configured = true;
   }
   const int rounds = (p.unit_splits + 7) / 8;
   const unsigned grid = (unsigned)(rounds * 8 * p.members);
-  hipLaunchKernelGGL((attn_ring_kernel<M, DH, NQB>), dim3(grid), dim3(256), lds, stream, p);
+  hipLaunchKernelGGL((attn_ring_kernel<M, DH, KSPLIT>), dim3(grid), dim3(512), lds, stream, p);
   return hipGetLastError();
 }
 
-hipError_t launch_attn_ring(const AttnParams& p, int Dh, int dtype, int variant, hipStream_t stream) {
-  const bool big = variant == 2;
+hipError_t launch_attn_ring(const AttnParams& p, int Dh, int dtype, int ksplit, hipStream_t stream) {
   if (dtype == WE_DTYPE_BF16) {
-    if (Dh == 128) return big ? launch_attn_t<Bf16Mma, 128, 2>(p, stream) : launch_attn_t<Bf16Mma, 128, 1>(p, stream);
-    if (Dh == 64) return big ? launch_attn_t<Bf16Mma, 64, 2>(p, stream) : launch_attn_t<Bf16Mma, 64, 1>(p, stream);
+    if (Dh == 128) return ksplit == 2 ? launch_ring_t<Bf16Mma, 128, 2>(p, stream) : launch_ring_t<Bf16Mma, 128, 1>(p, stream);
+    if (Dh == 64) return ksplit == 2 ? launch_ring_t<Bf16Mma, 64, 2>(p, stream) : launch_ring_t<Bf16Mma, 64, 1>(p, stream);
   } else if (dtype == WE_DTYPE_F16) {
-    if (Dh == 128) return big ? launch_attn_t<F16Mma, 128, 2>(p, stream) : launch_attn_t<F16Mma, 128, 1>(p, stream);
-    if (Dh == 64) return big ? launch_attn_t<F16Mma, 64, 2>(p, stream) : launch_attn_t<F16Mma, 64, 1>(p, stream);
+    if (Dh == 128) return ksplit == 2 ? launch_ring_t<F16Mma, 128, 2>(p, stream) : launch_ring_t<F16Mma, 128, 1>(p, stream);
+    if (Dh == 64) return ksplit == 2 ? launch_ring_t<F16Mma, 64, 2>(p, stream) : launch_ring_t<F16Mma, 64, 1>(p, stream);
   }
   return hipErrorInvalidValue;
-}
-
-hipError_t launch_attn_combine(const AttnParams& p, int Dh, int dtype, hipStream_t stream) {
-  const int64_t total = ((int64_t)p.B * p.H * p.T - p.ws_row0) * (Dh / 8);
-  const unsigned grid = (unsigned)((total + 255) / 256);
-  if (dtype == WE_DTYPE_BF16) {
-    if (Dh == 128) hipLaunchKernelGGL((attn_combine_kernel<Bf16Mma, 128>), dim3(grid), dim3(256), 0, stream, p);
-    else hipLaunchKernelGGL((attn_combine_kernel<Bf16Mma, 64>), dim3(grid), dim3(256), 0, stream, p);
-  } else {
-    if (Dh == 128) hipLaunchKernelGGL((attn_combine_kernel<F16Mma, 128>), dim3(grid), dim3(256), 0, stream, p);
-    else hipLaunchKernelGGL((attn_combine_kernel<F16Mma, 64>), dim3(grid), dim3(256), 0, stream, p);
-  }
-  return hipGetLastError();
 }
 
 }  // namespace we

@@ -22,7 +22,7 @@ int ring_shape_ok(int B, int H, int Hkv, int T, int Dh, int64_t L, int dilation)
 }
 
 struct AttnPlan {
-  int variant;      // 1/2: 4-wavefront kernel with 128/256 queries; 3/4: 8-wavefront kernel with 128/256
+  int variant;      // 1: 128 queries per workgroup, 2: 256
   int block_m;      // queries per workgroup
   int n_splits;     // context splits of the units that are split (1: none)
   int units_whole;  // leading (batch, kv head) units that are not split
@@ -30,8 +30,8 @@ struct AttnPlan {
 };
 
 // Pick the kernel shape and the context splitting.
-//  * Shape: the 8-wavefront kernel, 256 queries per workgroup when that alone gives at least one
-//    workgroup per CU, else 128 queries.
+//  * Shape: 256 queries per workgroup when that alone gives at least one workgroup per CU, else
+//    128 queries (two wavefronts share each query block and split every tile's keys).
 //  * Few workgroups (256-token frames): every unit is split into the same number of context
 //    parts, enough for one workgroup per CU but never fewer than two 64-key tiles per part.
 //  * Many workgroups that do not divide into whole rounds of 256 CUs (e.g. 384): only the units
@@ -39,8 +39,8 @@ struct AttnPlan {
 AttnPlan plan_attn(int B, int H, int Hkv, int T, int64_t L, int n_splits, int variant) {
   AttnPlan pl;
   const int64_t wg256 = (int64_t)B * H * ((T + 255) / 256);
-  pl.variant = variant ? variant : ((T >= 256 && wg256 >= 256) ? 4 : 3);
-  pl.block_m = (pl.variant == 2 || pl.variant == 4) ? 256 : 128;
+  pl.variant = variant ? variant : ((T >= 256 && wg256 >= 256) ? 2 : 1);
+  pl.block_m = pl.variant == 2 ? 256 : 128;
   const int units = B * Hkv;
   const int members = (H / Hkv) * ((T + pl.block_m - 1) / pl.block_m);
   const int64_t wgs = (int64_t)units * members;
@@ -77,8 +77,6 @@ int variant_of(int q_tile) {
     case 0: return 0;
     case 128: return 1;
     case 256: return 2;
-    case 129: return 3;
-    case 257: return 4;
     default: return -1;
   }
 }
@@ -226,9 +224,7 @@ int we_attn_ring_fwd(const void* q, const int64_t q_strides[3], const void* kv, 
   p.scale_log2 = scale * 1.4426950408889634f;
 
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const hipError_t le = pl.variant >= 3 ? we::launch_attn_ring8(p, Dh, dtype, pl.variant == 3 ? 2 : 1, st)
-                                        : we::launch_attn_ring(p, Dh, dtype, pl.variant, st);
-  if (le != hipSuccess) return WE_ERR_LAUNCH;
+  if (we::launch_attn_ring(p, Dh, dtype, pl.variant == 1 ? 2 : 1, st) != hipSuccess) return WE_ERR_LAUNCH;
   if (pl.n_splits > 1 && we::launch_attn_combine(p, Dh, dtype, st) != hipSuccess) return WE_ERR_LAUNCH;
   return WE_OK;
 }

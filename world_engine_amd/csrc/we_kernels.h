@@ -53,10 +53,8 @@ struct AttnParams {
 
 hipError_t launch_rope_kv_store(const StoreParams& p, int dtype, hipStream_t stream);
 
-// 4-wavefront kernel: variant 1 -> 128 queries per workgroup, 2 -> 256
-hipError_t launch_attn_ring(const AttnParams& p, int Dh, int dtype, int variant, hipStream_t stream);
-// 8-wavefront LDS-DMA kernel: groups = 2 -> 128 queries per workgroup, 1 -> 256
-hipError_t launch_attn_ring8(const AttnParams& p, int Dh, int dtype, int groups, hipStream_t stream);
+// main kernel: ksplit = 2 -> 128 queries per workgroup, 1 -> 256
+hipError_t launch_attn_ring(const AttnParams& p, int Dh, int dtype, int ksplit, hipStream_t stream);
 hipError_t launch_attn_combine(const AttnParams& p, int Dh, int dtype, hipStream_t stream);
 
 }  // namespace we
