@@ -27,6 +27,12 @@ if ROOT not in sys.path:
 PEAK_HBM_GBPS = 8000.0       # MI355X HBM3E, published
 PEAK_BF16_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
 
+# HBM-side bytes per attention call (attn_ring_kernel + attn_combine_kernel, reads + writes) from
+# two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) with the library's own split/tile choice, each
+# scaled by the same counter's reading for a 256 MiB copy kernel (FETCH_SIZE x2.000, WRITE_SIZE
+# x1.000); the summaries are profiles/attn_ring_cfg{1,3}_hbm_traffic.txt.
+MEASURED_TRAFFIC = {1: 63849600, 3: 505971744}
+
 CONFIGS = {
     1: dict(name="cfg1: B=1 H=16 Dh=128 T=256 16-slot ring (4096-token context) bf16, steady-state wrap",
             B=1, H=16, Hkv=16, Dh=128, T=256, slots=16, layers=1, frozen_subs=0, bound="hbm"),
@@ -63,6 +69,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--attn-iters", type=int, default=200, help="attention-only launches for the roofline timing")
     ap.add_argument("--batch", type=int, default=0, help="override the configuration's batch size (experiments)")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
+                    help="also launch 20 plain copy kernels (read MiB, write MiB each) so a counter run holds "
+                         "a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
     args = ap.parse_args()
 
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -131,6 +140,19 @@ def main():
                                       layer.kv, layer.written, layer.L, 1, frozen)
             ops.attn_ring(q_rot, layer.kv, layer.written, pos["t_pos"], layer.L, 1, n_splits=args.n_splits,
                           q_tile=args.q_tile, out=out, workspace=ws)
+
+    if args.calibrate_copy:
+        # elementwise copy through a kernel (a same-dtype copy_() could take the DMA engines and
+        # would then be invisible to the shader counters); int32 + 0 keeps the bytes unchanged
+        n_el = args.calibrate_copy * (1 << 20) // 4
+        src = torch.arange(n_el, dtype=torch.int32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(20):
+            torch.add(src, 0, out=dst)
+        torch.cuda.synchronize()
+        assert torch.equal(src[-4096:], dst[-4096:])
+        log(f"[bench] calibration: 20 copy kernels of {args.calibrate_copy} MiB read + {args.calibrate_copy} MiB written")
+        del src, dst
 
     # ---- fill the ring (untimed, not counted), then W warm-up steps ----
     fill_steps = n * subs
@@ -210,6 +232,8 @@ def main():
     else:
         roof = {"bound": "mfma", "achieved": round(tflops, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(tflops / PEAK_BF16_TFLOPS, 4), "traffic": None}
+    if not (args.n_splits or args.q_tile or args.batch):
+        roof["traffic"] = MEASURED_TRAFFIC.get(args.config)
     roof.update({"kernel": "attn_ring_kernel" + (" + attn_combine_kernel" if n_splits > 1 else ""),
                  "us_per_launch": round(attn_us, 3), "algorithmic_bytes": byts, "algorithmic_flops": flops,
                  "n_splits": n_splits})
