@@ -47,7 +47,7 @@ struct RingLds {
   static constexpr int SLOTS = 4;             // ring slots per operand over all wave groups
   static constexpr int V_OFF = SLOTS * TILE_B;
   static constexpr int MISC_OFF = 2 * SLOTS * TILE_B;
-  static constexpr int kBytes = MISC_OFF + (WE_MAX_SLOTS + 2) * 4;
+  static constexpr int kBytes = MISC_OFF + 8 * (WE_MAX_SLOTS + 64) * 4;  // + a slot-list strip per wavefront
 };
 
 // chunk swizzles: physical 16-byte chunk = logical chunk ^ swz(row)
@@ -116,7 +116,6 @@ __global__ void __launch_bounds__(512, 2) attn_ring_kernel(AttnParams p) {
   constexpr int NDMA = TILE_B / 1024 / 8;   // DMA instructions per wavefront and tile operand
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  int* vis = reinterpret_cast<int*>(smem + L::MISC_OFF);  // visible slots, then their count
   const uint32_t lds0 =
       (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
 
@@ -125,11 +124,19 @@ __global__ void __launch_bounds__(512, 2) attn_ring_kernel(AttnParams p) {
   const int qb = wave % QW;   // query block of this wavefront
   const int hb = wave / QW;   // key block of every tile it handles when KSPLIT == 2 (else 0)
 
-  // ---- which (batch, head, query tile, split) this workgroup owns; XCD = blockIdx % 8 ----
-  const int xcd = blockIdx.x & 7, jj = blockIdx.x >> 3;
-  const int round = jj / p.members, member = jj - round * p.members;
-  const int us = round * 8 + xcd;
-  if (us >= p.unit_splits) return;
+  // ---- frame index and slot flags: they need nothing but the kernel arguments ----
+  const int64_t frame_t = p.t_pos[0];
+  uint8_t flag = lane < p.n_slots ? p.written[(int64_t)lane * p.T] : (uint8_t)0;
+
+  // ---- which (batch, head, query tile, split) this workgroup owns ----
+  // The grid is (8 * query tiles, query heads per kv head, rounds): workgroups are dispatched
+  // to XCDs round-robin in linear order, so XCD = blockIdx.x % 8, and the workgroups that share
+  // one K/V stream (the x * y of one round) all land on the same XCD and its L2.
+  const int xcd = blockIdx.x & 7, qtile = blockIdx.x >> 3, hq_in = blockIdx.y;
+  const int us_raw = blockIdx.z * 8 + xcd;
+  // a workgroup past the end computes the addresses of the last one and leaves further down, so
+  // that the requests above and below do not wait behind a branch
+  const int us = us_raw < p.unit_splits ? us_raw : p.unit_splits - 1;
   // leading units run unsplit; the rest are cut into n_splits context parts each
   int unit, split, nsp;
   if (us < p.units_whole) {
@@ -139,10 +146,9 @@ __global__ void __launch_bounds__(512, 2) attn_ring_kernel(AttnParams p) {
     unit = p.units_whole + r / p.n_splits; split = r % p.n_splits; nsp = p.n_splits;
   }
   const int b = unit / p.Hkv, hkv = unit - b * p.Hkv;
-  const int hq_in = member / p.q_tiles, qtile = member - hq_in * p.q_tiles;
-  const int h = hkv * (p.H / p.Hkv) + hq_in;
+  const int h = hkv * p.group + hq_in;
 
-  // ---- raw Q fragments: requested first so the loads overlap the slot-list construction ----
+  // ---- raw Q fragments ----
   frag_t qf[KS];
   const int qrow = qtile * BM + qb * 32 + l32;
   {
@@ -152,55 +158,40 @@ __global__ void __launch_bounds__(512, 2) attn_ring_kernel(AttnParams p) {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) qf[ks] = *reinterpret_cast<const frag_t*>(src + ks * 16);
   }
+  if (us_raw >= p.unit_splits) return;
 
   // ---- list of visible slots (the tail is pseudo-slot n_slots) ----
-  if (wave == 0) {
-    const SlotInfo si = ring_slot(p.t_pos[0], p.dilation, p.num_buckets);
-    int count = 0;
+  // Every wavefront builds it for itself (no barrier, no serial section) in a private strip of
+  // LDS: lane i of round k looks at slot 64*k + i.  Entries 0..63 then live in one register (lane
+  // i holds entry i), which is where the hot loop looks them up; longer lists fall back to LDS.
+  int* vis = reinterpret_cast<int*>(smem + L::MISC_OFF) + wave * (WE_MAX_SLOTS + 64);
+  int nvis = 0;
+  {
+    const SlotInfo si = ring_slot(frame_t, p.dilation, p.num_buckets);
     for (int base = 0; base < p.n_slots; base += 64) {
-      const int s = base + lane;
-      bool f = false;
-      if (s < p.n_slots) f = (p.written[(int64_t)s * p.T] != 0) && !(si.write_step && s == si.slot);
+      const int sl = base + lane;
+      const bool f = flag != 0 && !(si.write_step && sl == si.slot);
+      if (base + 64 < p.n_slots) flag = sl + 64 < p.n_slots ? p.written[(int64_t)(sl + 64) * p.T] : (uint8_t)0;
       const unsigned long long m = __ballot(f);
-      if (f) vis[count + __popcll(m & ((1ull << lane) - 1ull))] = s;
-      count += __popcll(m);
+      if (f) vis[nvis + __popcll(m & ((1ull << lane) - 1ull))] = sl;
+      nvis += __popcll(m);
     }
-    if (lane == 0) {
-      vis[count] = p.n_slots;
-      vis[WE_MAX_SLOTS + 1] = count + 1;
-    }
+    if (lane == 0) vis[nvis] = p.n_slots;
+    ++nvis;
   }
-  __syncthreads();
-  const int nvis = __builtin_amdgcn_readfirstlane(vis[WE_MAX_SLOTS + 1]);
-  // The list moves into registers (entry i in lane i % 64 of register i / 64) so that the hot
-  // loop can look slots up with v_readlane instead of an LDS read it would have to wait for.
-  int visr[(WE_MAX_SLOTS + 64) / 64];
-#pragma unroll
-  for (int k = 0; k < (WE_MAX_SLOTS + 64) / 64; ++k) visr[k] = (64 * k + lane < nvis) ? vis[64 * k + lane] : 0;
+  const int vis0 = lane < nvis ? vis[lane] : 0;
   auto vis_at = [&](int i) __attribute__((always_inline)) {
-    const int l = i & 63;
-    switch (i >> 6) {
-      case 0: return __builtin_amdgcn_readlane(visr[0], l);
-      case 1: return __builtin_amdgcn_readlane(visr[1], l);
-      case 2: return __builtin_amdgcn_readlane(visr[2], l);
-      case 3: return __builtin_amdgcn_readlane(visr[3], l);
-      default: return __builtin_amdgcn_readlane(visr[4], l);
-    }
+    if (__builtin_expect(i < 64, 1)) return __builtin_amdgcn_readlane(vis0, i);
+    return __builtin_amdgcn_readfirstlane(vis[i]);
   };
   const int tps = p.T / BN;  // tiles per slot
   const int nt = nvis * tps;
-  const int t_begin = (int)((int64_t)split * nt / nsp);
-  const int t_end = (int)((int64_t)(split + 1) * nt / nsp);
-  const int ntile = t_end - t_begin;
-
-  // ---- Q stays in registers for the whole kernel, pre-multiplied by scale*log2(e) ----
-  const float c2 = p.scale_log2;
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    const frag_t raw = qf[ks];
-    qf[ks] = M::pack8((float)raw[0] * c2, (float)raw[1] * c2, (float)raw[2] * c2, (float)raw[3] * c2,
-                      (float)raw[4] * c2, (float)raw[5] * c2, (float)raw[6] * c2, (float)raw[7] * c2);
+  int t_begin = 0, t_end = nt;
+  if (nsp > 1) {  // nt <= 257 * T / 64 and nsp <= 64: the products fit 32 bits
+    t_begin = (int)((unsigned)split * (unsigned)nt / (unsigned)nsp);
+    t_end = (int)((unsigned)(split + 1) * (unsigned)nt / (unsigned)nsp);
   }
+  const int ntile = t_end - t_begin;
 
   const int64_t cap = p.L + p.T;
   const uint64_t kbase = (uint64_t)(uintptr_t)p.kv + (uint64_t)(((int64_t)b * p.Hkv + hkv) * cap) * ROW_B;
@@ -459,6 +450,10 @@ __global__ void __launch_bounds__(512, 2) attn_ring_kernel(AttnParams p) {
     // The V stream trails the K stream by KA - 2 tiles, so it reuses the K stream's offsets.
     TileWalk kw = walk_init();
     uint32_t off1, off2;  // offsets of the last and the last-but-one tile the K stream visited
+    // Q was requested before the slot flags and loads return in order, so it is here; stating a
+    // use now keeps the wait for it from landing behind the tile DMAs issued next.
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) asm volatile("" ::"v"(qf[ks]));
     {
       const uint32_t o0 = tile_off(kw); walk_next(kw);
       const uint32_t o1 = tile_off(kw); walk_next(kw);
@@ -476,6 +471,15 @@ __global__ void __launch_bounds__(512, 2) attn_ring_kernel(AttnParams p) {
         off1 = o3; off2 = o2;
       }
       dma_v(o1, 1);
+    }
+    // ---- Q stays in registers for the whole kernel, pre-multiplied by scale*log2(e); done while
+    //      the first tiles are on their way ----
+    const float c2 = p.scale_log2;
+  #pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const frag_t raw = qf[ks];
+      qf[ks] = M::pack8((float)raw[0] * c2, (float)raw[1] * c2, (float)raw[2] * c2, (float)raw[3] * c2,
+                        (float)raw[4] * c2, (float)raw[5] * c2, (float)raw[6] * c2, (float)raw[7] * c2);
     }
     dma_wait<(KA + 1) * NDMA>();
     __syncthreads();  // K(0) and the zeroed V slot are in LDS
@@ -643,8 +647,8 @@ static hipError_t launch_ring_t(const AttnParams& p, hipStream_t stream) {
     configured = true;
   }
   const int rounds = (p.unit_splits + 7) / 8;
-  const unsigned grid = (unsigned)(rounds * 8 * p.members);
-  hipLaunchKernelGGL((attn_ring_kernel<M, DH, KSPLIT>), dim3(grid), dim3(512), lds, stream, p);
+  const dim3 grid((unsigned)(8 * p.q_tiles), (unsigned)p.group, (unsigned)rounds);
+  hipLaunchKernelGGL((attn_ring_kernel<M, DH, KSPLIT>), grid, dim3(512), lds, stream, p);
   return hipGetLastError();
 }
 

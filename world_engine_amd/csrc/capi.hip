@@ -219,10 +219,12 @@ int we_attn_ring_fwd(const void* q, const int64_t q_strides[3], const void* kv, 
   p.units_whole = pl.units_whole;
   p.ws_row0 = (int64_t)B * H * T - pl.ws_rows;
   p.q_tiles = (T + pl.block_m - 1) / pl.block_m;
-  p.members = (H / Hkv) * p.q_tiles;
+  p.group = H / Hkv;
+  p.members = p.group * p.q_tiles;
   p.unit_splits = pl.units_whole + (B * Hkv - pl.units_whole) * pl.n_splits;
   p.scale_log2 = scale * 1.4426950408889634f;
 
+  if ((p.unit_splits + 7) / 8 > 65535 || p.group > 65535) return WE_ERR_UNSUPPORTED;  // grid z / y limits
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (we::launch_attn_ring(p, Dh, dtype, pl.variant == 1 ? 2 : 1, st) != hipSuccess) return WE_ERR_LAUNCH;
   if (pl.n_splits > 1 && we::launch_attn_combine(p, Dh, dtype, st) != hipSuccess) return WE_ERR_LAUNCH;

@@ -31,6 +31,21 @@ struct SlotInfo {
 };
 __device__ __forceinline__ SlotInfo ring_slot(int64_t frame_t, int dilation, int num_buckets) {
   SlotInfo s;
+  // Frame indices are small and non-negative in practice: 32-bit unsigned arithmetic, a fraction
+  // of the instructions of the emulated 64-bit signed divisions (kernels are launched once per
+  // layer and frame, so their straight-line start-up code is paid for by instruction fetch).
+  if (__builtin_expect((uint64_t)frame_t < 0x7fff0000ull && dilation > 0 && dilation < 0x10000, 1)) {
+    const uint32_t t = (uint32_t)frame_t;
+    if (dilation == 1) {
+      s.slot = (int)(t % (uint32_t)num_buckets);
+      s.write_step = true;
+    } else {
+      const uint32_t bucket = (t + (uint32_t)dilation - 1u) / (uint32_t)dilation;
+      s.slot = (int)(bucket % (uint32_t)num_buckets);
+      s.write_step = t % (uint32_t)dilation == 0u;
+    }
+    return s;
+  }
   int64_t bucket = floor_div(frame_t + (dilation - 1), (int64_t)dilation);
   s.slot = (int)floor_mod(bucket, (int64_t)num_buckets);
   s.write_step = floor_mod(frame_t, (int64_t)dilation) == 0;

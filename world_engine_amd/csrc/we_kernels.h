@@ -46,7 +46,8 @@ struct AttnParams {
   int units_whole;  // leading (batch, kv head) units processed unsplit, writing the output directly
   int64_t ws_row0;  // first query row covered by the split-context workspace
   int q_tiles;      // ceil(T / queries per workgroup)
-  int members;      // workgroups that share one K/V stream: (H/Hkv) * q_tiles
+  int group;        // query heads per kv head, H / Hkv
+  int members;      // workgroups that share one K/V stream: group * q_tiles
   int unit_splits;  // units_whole + (B * Hkv - units_whole) * n_splits
   float scale_log2; // softmax scale * log2(e)
 };
