@@ -10,15 +10,17 @@ namespace we {
 
 // Second pass of the split-context path.  Every split left, per query row, its normalised
 // output O_s (element type), its reference m_s (log2 domain) and its sum l_s; the result is
-// sum_s w_s O_s / sum_s w_s with w_s = 2^(m_s - max m) * l_s.  One thread per (row, 8 columns).
+// sum_s w_s O_s / sum_s w_s with w_s = 2^(m_s - max m) * l_s.  One thread per (row, 8 columns);
+// grid = (256-thread slices of one head's T * DH/8 items, split (batch, head) pairs), so that the
+// start-up code has one 32-bit division in it (the kernel is short enough for that to show).
 template <typename M, int DH>
 __global__ void __launch_bounds__(256) attn_combine_kernel(AttnParams p) {
   typedef typename M::frag_t frag_t;
   const int64_t rows = (int64_t)p.B * p.H * p.T - p.ws_row0;  // rows that were split
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= rows * (DH / 8)) return;
-  const int64_t row = idx / (DH / 8);  // workspace row; query row = row + ws_row0
-  const int dg = (int)(idx % (DH / 8));
+  const int item = blockIdx.x * 256 + threadIdx.x;
+  if (item >= p.T * (DH / 8)) return;
+  const int t = item / (DH / 8), dg = item % (DH / 8);
+  const int64_t row = (int64_t)blockIdx.y * p.T + t;  // workspace row; query row = row + ws_row0
   // Splits are merged eight at a time with all sixteen loads of a batch issued before the first
   // use (a plain loop over a run-time split count would serialise one memory round trip per split).
   float mmax = -INFINITY, den = 0.f;
@@ -51,19 +53,15 @@ __global__ void __launch_bounds__(256) attn_combine_kernel(AttnParams p) {
     mmax = bmax;
   }
   const float inv = 1.f / den;
-  const int64_t qrow = row + p.ws_row0;
-  const int t = (int)(qrow % p.T);
-  const int64_t bh = qrow / p.T;
-  const int h = (int)(bh % p.H);
-  const int b = (int)(bh / p.H);
+  const unsigned bh = (unsigned)(p.units_whole * p.group) + blockIdx.y;  // first split pair + y
+  const int b = (int)(bh / (unsigned)p.H), h = (int)(bh % (unsigned)p.H);
   uint16_t* dst = reinterpret_cast<uint16_t*>(p.out) + b * p.os_b + h * p.os_h + (int64_t)t * p.os_t + dg * 8;
   *reinterpret_cast<frag_t*>(dst) = M::pack8(acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv, acc[4] * inv,
                                              acc[5] * inv, acc[6] * inv, acc[7] * inv);
 }
 
 hipError_t launch_attn_combine(const AttnParams& p, int Dh, int dtype, hipStream_t stream) {
-  const int64_t total = ((int64_t)p.B * p.H * p.T - p.ws_row0) * (Dh / 8);
-  const unsigned grid = (unsigned)((total + 255) / 256);
+  const dim3 grid((unsigned)((p.T * (Dh / 8) + 255) / 256), (unsigned)(p.B * p.H - p.units_whole * p.group));
   if (dtype == WE_DTYPE_BF16) {
     if (Dh == 128) hipLaunchKernelGGL((attn_combine_kernel<Bf16Mma, 128>), dim3(grid), dim3(256), 0, stream, p);
     else hipLaunchKernelGGL((attn_combine_kernel<Bf16Mma, 64>), dim3(grid), dim3(256), 0, stream, p);

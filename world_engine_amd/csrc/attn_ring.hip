@@ -573,26 +573,32 @@ __global__ void __launch_bounds__(512, 2) attn_ring_kernel(AttnParams p) {
 
   if (KSPLIT == 2) {
     // ---- the two wavefronts of a query block merge their (m, l, O) through LDS ----
+    // 16-byte accesses: vector k of lane l sits at ((qb * (DB * 4 + 1) + k) * 64 + l) * 16.
     __syncthreads();  // every wavefront is done with the rings
-    float* mb = reinterpret_cast<float*>(smem) + (qb * (DB * 16 + 2)) * 64 + lane;
+    f32x4_t* mb = reinterpret_cast<f32x4_t*>(smem) + (qb * (DB * 4 + 1)) * 64 + lane;
     if (hb == 1) {
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) mb[(db * 16 + i) * 64] = o[db][i];
-      mb[(DB * 16) * 64] = m_ref;
-      mb[(DB * 16 + 1) * 64] = l_tot;
+        for (int c = 0; c < 4; ++c)
+          mb[(db * 4 + c) * 64] = f32x4_t{o[db][4 * c], o[db][4 * c + 1], o[db][4 * c + 2], o[db][4 * c + 3]};
+      mb[(DB * 4) * 64] = f32x4_t{m_ref, l_tot, 0.f, 0.f};
     }
     __syncthreads();
     if (hb == 1) return;
-    const float m1 = mb[(DB * 16) * 64], l1 = mb[(DB * 16 + 1) * 64];
+    const f32x4_t ml1 = mb[(DB * 4) * 64];
+    const float m1 = ml1[0], l1 = ml1[1];
     const float mm = fmaxf(m_ref, m1);
     if (mm > -INFINITY) {
       const float a0 = __builtin_amdgcn_exp2f(m_ref - mm), a1 = __builtin_amdgcn_exp2f(m1 - mm);
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) o[db][i] = a0 * o[db][i] + a1 * mb[(db * 16 + i) * 64];
+        for (int c = 0; c < 4; ++c) {
+          const f32x4_t other = mb[(db * 4 + c) * 64];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o[db][4 * c + e] = a0 * o[db][4 * c + e] + a1 * other[e];
+        }
       l_tot = a0 * l_tot + a1 * l1;
       m_ref = mm;
     }

@@ -133,6 +133,9 @@ int we_rope_kv_store(const void* q, const void* k, const void* v, const int64_t 
   p.pos_stride_b = pos_stride_b;
   p.table_rows = table_rows;
   p.grid_hw = grid_h * grid_w; p.grid_w = grid_w;
+  p.cpr_shift = -1;
+  for (int sh = 0; sh < 16; ++sh)
+    if ((Dh >> 4) == (1 << sh)) p.cpr_shift = sh;
   p.L = L;
   p.B = B; p.H = H; p.Hkv = Hkv; p.T = T; p.Dh = Dh;
   p.dilation = dilation; p.num_buckets = (int)((L / T) / dilation); p.frozen = is_frozen ? 1 : 0;
@@ -160,6 +163,9 @@ int we_rope_apply(const void* x, const int64_t x_strides[3], void* x_out, const 
   p.pos_stride_b = pos_stride_b;
   p.table_rows = table_rows;
   p.grid_hw = grid_h * grid_w; p.grid_w = grid_w;
+  p.cpr_shift = -1;
+  for (int sh = 0; sh < 16; ++sh)
+    if ((Dh >> 4) == (1 << sh)) p.cpr_shift = sh;
   p.L = T;
   p.B = B; p.H = H; p.Hkv = 0; p.T = T; p.Dh = Dh;
   p.dilation = 1; p.num_buckets = 1; p.frozen = 1;
@@ -224,7 +230,8 @@ int we_attn_ring_fwd(const void* q, const int64_t q_strides[3], const void* kv, 
   p.unit_splits = pl.units_whole + (B * Hkv - pl.units_whole) * pl.n_splits;
   p.scale_log2 = scale * 1.4426950408889634f;
 
-  if ((p.unit_splits + 7) / 8 > 65535 || p.group > 65535) return WE_ERR_UNSUPPORTED;  // grid z / y limits
+  if ((p.unit_splits + 7) / 8 > 65535 || p.group > 65535 || (int64_t)B * H - (int64_t)pl.units_whole * p.group > 65535)
+    return WE_ERR_UNSUPPORTED;  // grid y / z limits of the two launches
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (we::launch_attn_ring(p, Dh, dtype, pl.variant == 1 ? 2 : 1, st) != hipSuccess) return WE_ERR_LAUNCH;
   if (pl.n_splits > 1 && we::launch_attn_combine(p, Dh, dtype, st) != hipSuccess) return WE_ERR_LAUNCH;

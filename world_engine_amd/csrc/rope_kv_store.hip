@@ -84,7 +84,7 @@ __global__ void __launch_bounds__(256) rope_kv_store_kernel(StoreParams p) {
   const int hkv = p.k ? p.Hkv : 0;  // rotation-only launches carry no k/v
   const int idx = blockIdx.x * 256 + threadIdx.x;
   if (idx >= p.T * cpr) return;
-  const int t = idx / cpr;
+  const int t = p.cpr_shift >= 0 ? idx >> p.cpr_shift : idx / cpr;  // head dims are powers of two in practice
   const int chunk = idx - t * cpr;
   const int head_all = blockIdx.y;
   const int b = blockIdx.z;

@@ -27,6 +27,7 @@ struct StoreParams {
   int64_t L;
   int B, H, Hkv, T, Dh;
   int dilation, num_buckets, frozen;
+  int cpr_shift;  // log2(Dh / 16) when Dh / 16 is a power of two, else -1
 };
 
 struct AttnParams {
