@@ -370,6 +370,19 @@ __global__ void __launch_bounds__(512, 2) attn_ring_kernel(AttnParams p) {
     frag_t p_cur[2];
     float e[16];
     float rs = 0.f;
+    // VALU slices: the 16 exponentials of the current block are spread evenly over the MFMAs of
+    // the step (slot 0 follows the shift product, slots 1..KS the logits, the rest the product).
+    // The two wavefronts of a SIMD run in phase, so bunching them under the logits would saturate
+    // the quarter-rate unit there and leave it idle under the product.
+    constexpr int EPS = 16 / (KS + NV);
+    static_assert(EPS * (KS + NV) == 16, "exponentials per slot");
+    auto exp_slot = [&](int g) __attribute__((always_inline)) {
+#pragma unroll
+      for (int t = 0; t < EPS; ++t)
+        if (g * EPS + t < 16) e[g * EPS + t] = __builtin_amdgcn_exp2f(s_cur[g * EPS + t]);
+    };
+    exp_slot(0);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       s_next = M::mma(__builtin_bit_cast(frag_t, kf[ks]), qf[ks], s_next);
@@ -379,10 +392,7 @@ __global__ void __launch_bounds__(512, 2) attn_ring_kernel(AttnParams p) {
         ++vnext;
         issued += 2;
       }
-      // VALU slice: 16 / KS exponentials of the current block
-#pragma unroll
-      for (int t = 0; t < 16 / KS; ++t)
-        e[ks * (16 / KS) + t] = __builtin_amdgcn_exp2f(s_cur[ks * (16 / KS) + t]);
+      exp_slot(1 + ks);
       __builtin_amdgcn_sched_barrier(0);
     }
     mid();  // the tile DMAs of this iteration go out here, under the MFMAs already queued
@@ -398,19 +408,18 @@ __global__ void __launch_bounds__(512, 2) attn_ring_kernel(AttnParams p) {
       const u32x4v a4 = __builtin_shufflevector(v0[i], v1[i], 0, 1, 2, 3);
       o[i % DB] = M::mma(__builtin_bit_cast(frag_t, a4), p_prev[i / DB], o[i % DB]);
       if (i >= I0 && npair < NPAIR) next_pair();
-      // VALU slices: pack the two 16-key halves, then their row sums
-      if (i == 0) p_cur[0] = M::pack8(e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7]);
-      if (i == 1) {
+      // VALU slices: the last exponentials; packing of the two 16-key halves and their row sums
+      exp_slot(1 + KS + i);
+      if (i == 1) p_cur[0] = M::pack8(e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7]);
+      if (i == 2) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) rs = M::add_pair(rs, p_cur[0], t);
       }
-      if (i == 2) p_cur[1] = M::pack8(e[8], e[9], e[10], e[11], e[12], e[13], e[14], e[15]);
-      if (i == 3) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t) rs = M::add_pair(rs, p_cur[1], t);
-      }
+      if (i == NV - 1) p_cur[1] = M::pack8(e[8], e[9], e[10], e[11], e[12], e[13], e[14], e[15]);
       __builtin_amdgcn_sched_barrier(0);
     }
+#pragma unroll
+    for (int t = 0; t < 4; ++t) rs = M::add_pair(rs, p_cur[1], t);
 
     if (__ballot(!(rs <= 256.f)) != 0ull) {
       // Rare: some probability of this block may exceed 2^8.  Raise the reference of the rows
