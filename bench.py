@@ -67,6 +67,8 @@ def main():
     ap.add_argument("--q-tile", type=int, default=0, help="queries per workgroup (0 = library's choice)")
     ap.add_argument("--eager", action="store_true", help="launch from Python per call instead of a HIP graph")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--two-calls", action="store_true",
+                    help="we_rope_kv_store + we_attn_ring_fwd instead of the one-call we_rope_kv_attn_fwd")
     ap.add_argument("--attn-iters", type=int, default=200, help="attention-only launches for the roofline timing")
     ap.add_argument("--batch", type=int, default=0, help="override the configuration's batch size (experiments)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
@@ -136,10 +138,15 @@ def main():
         pos = {"t_pos": t_pos_all[frame], "y_pos": y_pos, "x_pos": x_pos}
         for li, layer in enumerate(cache.layers):
             q, k, v = inputs[(step_idx + li) % n_in]
-            q_rot = ops.rope_kv_store(q, k, v, pos, rope.cos, rope.sin, rope.height, rope.width,
-                                      layer.kv, layer.written, layer.L, 1, frozen)
-            ops.attn_ring(q_rot, layer.kv, layer.written, pos["t_pos"], layer.L, 1, n_splits=args.n_splits,
-                          q_tile=args.q_tile, out=out, workspace=ws)
+            if args.two_calls:
+                q_rot = ops.rope_kv_store(q, k, v, pos, rope.cos, rope.sin, rope.height, rope.width,
+                                          layer.kv, layer.written, layer.L, 1, frozen)
+                ops.attn_ring(q_rot, layer.kv, layer.written, pos["t_pos"], layer.L, 1, n_splits=args.n_splits,
+                              q_tile=args.q_tile, out=out, workspace=ws)
+            else:
+                ops.rope_kv_attn(q, k, v, pos, rope.cos, rope.sin, rope.height, rope.width, layer.kv,
+                                 layer.written, layer.L, 1, frozen, n_splits=args.n_splits, q_tile=args.q_tile,
+                                 out=out, workspace=ws)
 
     if args.calibrate_copy:
         # elementwise copy through a kernel (a same-dtype copy_() could take the DMA engines and

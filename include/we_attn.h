@@ -150,6 +150,28 @@ int we_attn_ring_fwd(const void* q, const int64_t q_strides[3],
                      int32_t dilation, float scale, int32_t n_splits, int32_t q_tile,
                      int32_t dtype, void* stream);
 
+/*
+ * RoPE + K/V store + attention of one frame in a single call: we_rope_kv_store followed by
+ * we_attn_ring_fwd on the rotated q, i.e. the whole per-layer sequence of the reference from
+ * `q, k = rope(q), rope(k)` to the flex_attention call (src/model/attn.py:110-116 with
+ * src/model/kv_cache.py:126-151).  Arguments, requirements and results (cache rows, `written`,
+ * q_out, out) are those of the two calls, bit for bit; q, q_out and the tables are mandatory.
+ * Both calls are validated before anything is launched, and a host language pays for one
+ * foreign call per layer and frame instead of two.
+ */
+int we_rope_kv_attn_fwd(const void* q, const void* k, const void* v,
+                        const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                        void* q_out,
+                        const float* cos_table, const float* sin_table, int64_t table_rows,
+                        const int64_t* t_pos, const int64_t* y_pos, const int64_t* x_pos,
+                        int64_t pos_stride_b, int64_t grid_h, int64_t grid_w,
+                        void* kv, uint8_t* written,
+                        void* out, const int64_t out_strides[3],
+                        void* workspace, size_t workspace_bytes,
+                        int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L,
+                        int32_t dilation, int32_t is_frozen, float scale, int32_t n_splits, int32_t q_tile,
+                        int32_t dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

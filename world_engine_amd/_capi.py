@@ -50,6 +50,19 @@ SIGNATURES = {
         c_int32, c_int32, c_int32, c_int32, c_int32, c_int64,   # B H Hkv T Dh L
         c_int32, c_float, c_int32, c_int32, c_int32, c_void_p,  # dilation scale n_splits q_tile dtype stream
     ]),
+    "we_rope_kv_attn_fwd": (c_int32, [
+        c_void_p, c_void_p, c_void_p,              # q, k, v
+        _I64x3, _I64x3, _I64x3,                    # strides
+        c_void_p,                                  # q_out
+        c_void_p, c_void_p, c_int64,               # cos, sin, table_rows
+        c_void_p, c_void_p, c_void_p,              # t_pos, y_pos, x_pos
+        c_int64, c_int64, c_int64,                 # pos_stride_b, grid_h, grid_w
+        c_void_p, c_void_p,                        # kv, written
+        c_void_p, _I64x3,                          # out, out_strides
+        c_void_p, c_size_t,                        # workspace, bytes
+        c_int32, c_int32, c_int32, c_int32, c_int32, c_int64,   # B H Hkv T Dh L
+        c_int32, c_int32, c_float, c_int32, c_int32, c_int32, c_void_p,  # dilation frozen scale n_splits q_tile dtype stream
+    ]),
 }
 
 _lib = None

@@ -81,6 +81,93 @@ int variant_of(int q_tile) {
   }
 }
 
+// Validation of a we_rope_kv_store call and its kernel parameters.
+int prepare_store(const void* q, const void* k, const void* v, const int64_t* q_strides, const int64_t* k_strides,
+                  const int64_t* v_strides, void* q_out, const float* cos_table, const float* sin_table,
+                  int64_t table_rows, const int64_t* t_pos, const int64_t* y_pos, const int64_t* x_pos,
+                  int64_t pos_stride_b, int64_t grid_h, int64_t grid_w, void* kv, uint8_t* written, int B, int H,
+                  int Hkv, int T, int Dh, int64_t L, int dilation, int is_frozen, int dtype, we::StoreParams& p) {
+  if (!k || !v || !k_strides || !v_strides || !t_pos || !kv || !written) return WE_ERR_NULL_POINTER;
+  if ((q == nullptr) != (q_out == nullptr)) return WE_ERR_NULL_POINTER;
+  if (q && !q_strides) return WE_ERR_NULL_POINTER;
+  if ((cos_table == nullptr) != (sin_table == nullptr)) return WE_ERR_NULL_POINTER;
+  if (cos_table && (!y_pos || !x_pos)) return WE_ERR_NULL_POINTER;
+  if (dtype != WE_DTYPE_BF16 && dtype != WE_DTYPE_F16 && dtype != WE_DTYPE_F32) return WE_ERR_UNSUPPORTED;
+  int rc = ring_shape_ok(B, H, Hkv, T, Dh, L, dilation);
+  if (rc != WE_OK) return rc;
+  if (Dh % 16 != 0) return WE_ERR_UNSUPPORTED;
+  if (cos_table && (table_rows <= 0 || grid_h <= 0 || grid_w <= 0)) return WE_ERR_BAD_SHAPE;
+  if (!aligned16(k) || !aligned16(v) || !aligned16(kv) || (q && (!aligned16(q) || !aligned16(q_out))) ||
+      (cos_table && (!aligned16(cos_table) || !aligned16(sin_table))))
+    return WE_ERR_ALIGNMENT;
+  if (!strides_ok(k_strides, dtype) || !strides_ok(v_strides, dtype) || (q && !strides_ok(q_strides, dtype)))
+    return WE_ERR_ALIGNMENT;
+
+  p.q = q; p.k = k; p.v = v; p.q_out = q_out; p.kv = kv; p.written = written;
+  p.cos_t = cos_table; p.sin_t = sin_table;
+  p.t_pos = t_pos; p.y_pos = y_pos; p.x_pos = x_pos;
+  p.qs_b = q ? q_strides[0] : 0; p.qs_h = q ? q_strides[1] : 0; p.qs_t = q ? q_strides[2] : 0;
+  p.ks_b = k_strides[0]; p.ks_h = k_strides[1]; p.ks_t = k_strides[2];
+  p.vs_b = v_strides[0]; p.vs_h = v_strides[1]; p.vs_t = v_strides[2];
+  p.pos_stride_b = pos_stride_b;
+  p.table_rows = table_rows;
+  p.grid_hw = grid_h * grid_w; p.grid_w = grid_w;
+  p.cpr_shift = -1;
+  for (int sh = 0; sh < 16; ++sh)
+    if ((Dh >> 4) == (1 << sh)) p.cpr_shift = sh;
+  p.L = L;
+  p.B = B; p.H = H; p.Hkv = Hkv; p.T = T; p.Dh = Dh;
+  p.dilation = dilation; p.num_buckets = (int)((L / T) / dilation); p.frozen = is_frozen ? 1 : 0;
+  return WE_OK;
+}
+
+// Validation of a we_attn_ring_fwd call, its plan and its kernel parameters.
+int prepare_attn(const void* q, const int64_t* q_strides, const void* kv, const uint8_t* written,
+                 const int64_t* t_pos, void* out, const int64_t* out_strides, void* workspace, size_t workspace_bytes,
+                 int B, int H, int Hkv, int T, int Dh, int64_t L, int dilation, float scale, int n_splits, int q_tile,
+                 int dtype, we::AttnParams& p, AttnPlan& pl) {
+  if (!q || !q_strides || !kv || !written || !t_pos || !out || !out_strides) return WE_ERR_NULL_POINTER;
+  int rc = ring_shape_ok(B, H, Hkv, T, Dh, L, dilation);
+  if (rc != WE_OK) return rc;
+  if (dtype != WE_DTYPE_BF16 && dtype != WE_DTYPE_F16) return WE_ERR_UNSUPPORTED;
+  if (Dh != 64 && Dh != 128) return WE_ERR_UNSUPPORTED;
+  if (T % 64 != 0 || L / T > WE_MAX_SLOTS) return WE_ERR_UNSUPPORTED;
+  if ((uint64_t)(L + T) * (uint64_t)Dh * 2u >= (1ull << 32)) return WE_ERR_UNSUPPORTED;  // 32-bit tile offsets
+  if (!(scale > 0.f) || n_splits < 0 || n_splits > 64) return WE_ERR_BAD_SHAPE;
+  if (variant_of(q_tile) < 0) return WE_ERR_UNSUPPORTED;
+  if (!aligned16(q) || !aligned16(kv) || !aligned16(out) || !strides_ok(q_strides, dtype) ||
+      !strides_ok(out_strides, dtype))
+    return WE_ERR_ALIGNMENT;
+
+  pl = plan_attn(B, H, Hkv, T, L, n_splits, variant_of(q_tile));
+  const size_t ws_need = (size_t)pl.n_splits * (size_t)pl.ws_rows * ((size_t)Dh * 2 + 2 * sizeof(float));
+  if (ws_need > 0) {
+    if (!workspace || !aligned16(workspace)) return WE_ERR_WORKSPACE;
+    if (workspace_bytes < ws_need) return WE_ERR_WORKSPACE;
+  }
+
+  p.q = q; p.kv = kv; p.written = written; p.t_pos = t_pos; p.out = out;
+  p.ws_o = ws_need ? static_cast<uint16_t*>(workspace) : nullptr;
+  p.ws_ml = ws_need ? reinterpret_cast<float*>(p.ws_o + (size_t)pl.n_splits * (size_t)pl.ws_rows * Dh) : nullptr;
+  p.qs_b = q_strides[0]; p.qs_h = q_strides[1]; p.qs_t = q_strides[2];
+  p.os_b = out_strides[0]; p.os_h = out_strides[1]; p.os_t = out_strides[2];
+  p.L = L;
+  p.B = B; p.H = H; p.Hkv = Hkv; p.T = T;
+  p.n_slots = (int)(L / T); p.dilation = dilation; p.num_buckets = p.n_slots / dilation;
+  p.n_splits = pl.n_splits;
+  p.units_whole = pl.units_whole;
+  p.ws_row0 = (int64_t)B * H * T - pl.ws_rows;
+  p.q_tiles = (T + pl.block_m - 1) / pl.block_m;
+  p.group = H / Hkv;
+  p.members = p.group * p.q_tiles;
+  p.unit_splits = pl.units_whole + (B * Hkv - pl.units_whole) * pl.n_splits;
+  p.scale_log2 = scale * 1.4426950408889634f;
+
+  if ((p.unit_splits + 7) / 8 > 65535 || p.group > 65535 || (int64_t)B * H - (int64_t)pl.units_whole * p.group > 65535)
+    return WE_ERR_UNSUPPORTED;  // grid y / z limits of the two launches
+  return WE_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -107,38 +194,11 @@ int we_rope_kv_store(const void* q, const void* k, const void* v, const int64_t 
                      int64_t pos_stride_b, int64_t grid_h, int64_t grid_w, void* kv, uint8_t* written,
                      int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L,
                      int32_t dilation, int32_t is_frozen, int32_t dtype, void* stream) {
-  if (!k || !v || !k_strides || !v_strides || !t_pos || !kv || !written) return WE_ERR_NULL_POINTER;
-  if ((q == nullptr) != (q_out == nullptr)) return WE_ERR_NULL_POINTER;
-  if (q && !q_strides) return WE_ERR_NULL_POINTER;
-  if ((cos_table == nullptr) != (sin_table == nullptr)) return WE_ERR_NULL_POINTER;
-  if (cos_table && (!y_pos || !x_pos)) return WE_ERR_NULL_POINTER;
-  if (dtype != WE_DTYPE_BF16 && dtype != WE_DTYPE_F16 && dtype != WE_DTYPE_F32) return WE_ERR_UNSUPPORTED;
-  int rc = ring_shape_ok(B, H, Hkv, T, Dh, L, dilation);
-  if (rc != WE_OK) return rc;
-  if (Dh % 16 != 0) return WE_ERR_UNSUPPORTED;
-  if (cos_table && (table_rows <= 0 || grid_h <= 0 || grid_w <= 0)) return WE_ERR_BAD_SHAPE;
-  if (!aligned16(k) || !aligned16(v) || !aligned16(kv) || (q && (!aligned16(q) || !aligned16(q_out))) ||
-      (cos_table && (!aligned16(cos_table) || !aligned16(sin_table))))
-    return WE_ERR_ALIGNMENT;
-  if (!strides_ok(k_strides, dtype) || !strides_ok(v_strides, dtype) || (q && !strides_ok(q_strides, dtype)))
-    return WE_ERR_ALIGNMENT;
-
   we::StoreParams p;
-  p.q = q; p.k = k; p.v = v; p.q_out = q_out; p.kv = kv; p.written = written;
-  p.cos_t = cos_table; p.sin_t = sin_table;
-  p.t_pos = t_pos; p.y_pos = y_pos; p.x_pos = x_pos;
-  p.qs_b = q ? q_strides[0] : 0; p.qs_h = q ? q_strides[1] : 0; p.qs_t = q ? q_strides[2] : 0;
-  p.ks_b = k_strides[0]; p.ks_h = k_strides[1]; p.ks_t = k_strides[2];
-  p.vs_b = v_strides[0]; p.vs_h = v_strides[1]; p.vs_t = v_strides[2];
-  p.pos_stride_b = pos_stride_b;
-  p.table_rows = table_rows;
-  p.grid_hw = grid_h * grid_w; p.grid_w = grid_w;
-  p.cpr_shift = -1;
-  for (int sh = 0; sh < 16; ++sh)
-    if ((Dh >> 4) == (1 << sh)) p.cpr_shift = sh;
-  p.L = L;
-  p.B = B; p.H = H; p.Hkv = Hkv; p.T = T; p.Dh = Dh;
-  p.dilation = dilation; p.num_buckets = (int)((L / T) / dilation); p.frozen = is_frozen ? 1 : 0;
+  const int rc = prepare_store(q, k, v, q_strides, k_strides, v_strides, q_out, cos_table, sin_table, table_rows,
+                               t_pos, y_pos, x_pos, pos_stride_b, grid_h, grid_w, kv, written, B, H, Hkv, T, Dh,
+                               L, dilation, is_frozen, dtype, p);
+  if (rc != WE_OK) return rc;
   return we::launch_rope_kv_store(p, dtype, static_cast<hipStream_t>(stream)) == hipSuccess ? WE_OK : WE_ERR_LAUNCH;
 }
 
@@ -192,47 +252,42 @@ int we_attn_ring_fwd(const void* q, const int64_t q_strides[3], const void* kv, 
                      size_t workspace_bytes, int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh,
                      int64_t L, int32_t dilation, float scale, int32_t n_splits, int32_t q_tile,
                      int32_t dtype, void* stream) {
-  if (!q || !q_strides || !kv || !written || !t_pos || !out || !out_strides) return WE_ERR_NULL_POINTER;
-  int rc = ring_shape_ok(B, H, Hkv, T, Dh, L, dilation);
-  if (rc != WE_OK) return rc;
-  if (dtype != WE_DTYPE_BF16 && dtype != WE_DTYPE_F16) return WE_ERR_UNSUPPORTED;
-  if (Dh != 64 && Dh != 128) return WE_ERR_UNSUPPORTED;
-  if (T % 64 != 0 || L / T > WE_MAX_SLOTS) return WE_ERR_UNSUPPORTED;
-  if ((uint64_t)(L + T) * (uint64_t)Dh * 2u >= (1ull << 32)) return WE_ERR_UNSUPPORTED;  // 32-bit tile offsets
-  if (!(scale > 0.f) || n_splits < 0 || n_splits > 64) return WE_ERR_BAD_SHAPE;
-  if (variant_of(q_tile) < 0) return WE_ERR_UNSUPPORTED;
-  if (!aligned16(q) || !aligned16(kv) || !aligned16(out) || !strides_ok(q_strides, dtype) ||
-      !strides_ok(out_strides, dtype))
-    return WE_ERR_ALIGNMENT;
-
-  const AttnPlan pl = plan_attn(B, H, Hkv, T, L, n_splits, variant_of(q_tile));
-  const size_t ws_need = (size_t)pl.n_splits * (size_t)pl.ws_rows * ((size_t)Dh * 2 + 2 * sizeof(float));
-  if (ws_need > 0) {
-    if (!workspace || !aligned16(workspace)) return WE_ERR_WORKSPACE;
-    if (workspace_bytes < ws_need) return WE_ERR_WORKSPACE;
-  }
-
   we::AttnParams p;
-  p.q = q; p.kv = kv; p.written = written; p.t_pos = t_pos; p.out = out;
-  p.ws_o = ws_need ? static_cast<uint16_t*>(workspace) : nullptr;
-  p.ws_ml = ws_need ? reinterpret_cast<float*>(p.ws_o + (size_t)pl.n_splits * (size_t)pl.ws_rows * Dh) : nullptr;
-  p.qs_b = q_strides[0]; p.qs_h = q_strides[1]; p.qs_t = q_strides[2];
-  p.os_b = out_strides[0]; p.os_h = out_strides[1]; p.os_t = out_strides[2];
-  p.L = L;
-  p.B = B; p.H = H; p.Hkv = Hkv; p.T = T;
-  p.n_slots = (int)(L / T); p.dilation = dilation; p.num_buckets = p.n_slots / dilation;
-  p.n_splits = pl.n_splits;
-  p.units_whole = pl.units_whole;
-  p.ws_row0 = (int64_t)B * H * T - pl.ws_rows;
-  p.q_tiles = (T + pl.block_m - 1) / pl.block_m;
-  p.group = H / Hkv;
-  p.members = p.group * p.q_tiles;
-  p.unit_splits = pl.units_whole + (B * Hkv - pl.units_whole) * pl.n_splits;
-  p.scale_log2 = scale * 1.4426950408889634f;
-
-  if ((p.unit_splits + 7) / 8 > 65535 || p.group > 65535 || (int64_t)B * H - (int64_t)pl.units_whole * p.group > 65535)
-    return WE_ERR_UNSUPPORTED;  // grid y / z limits of the two launches
+  AttnPlan pl;
+  const int rc = prepare_attn(q, q_strides, kv, written, t_pos, out, out_strides, workspace, workspace_bytes, B, H,
+                              Hkv, T, Dh, L, dilation, scale, n_splits, q_tile, dtype, p, pl);
+  if (rc != WE_OK) return rc;
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (we::launch_attn_ring(p, Dh, dtype, pl.variant == 1 ? 2 : 1, st) != hipSuccess) return WE_ERR_LAUNCH;
+  if (pl.n_splits > 1 && we::launch_attn_combine(p, Dh, dtype, st) != hipSuccess) return WE_ERR_LAUNCH;
+  return WE_OK;
+}
+
+int we_rope_kv_attn_fwd(const void* q, const void* k, const void* v, const int64_t q_strides[3],
+                        const int64_t k_strides[3], const int64_t v_strides[3], void* q_out,
+                        const float* cos_table, const float* sin_table, int64_t table_rows,
+                        const int64_t* t_pos, const int64_t* y_pos, const int64_t* x_pos, int64_t pos_stride_b,
+                        int64_t grid_h, int64_t grid_w, void* kv, uint8_t* written, void* out,
+                        const int64_t out_strides[3], void* workspace, size_t workspace_bytes, int32_t B,
+                        int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L, int32_t dilation,
+                        int32_t is_frozen, float scale, int32_t n_splits, int32_t q_tile, int32_t dtype,
+                        void* stream) {
+  if (!q || !q_out || !cos_table) return WE_ERR_NULL_POINTER;
+  we::StoreParams sp;
+  int rc = prepare_store(q, k, v, q_strides, k_strides, v_strides, q_out, cos_table, sin_table, table_rows, t_pos,
+                         y_pos, x_pos, pos_stride_b, grid_h, grid_w, kv, written, B, H, Hkv, T, Dh, L, dilation,
+                         is_frozen, dtype, sp);
+  if (rc != WE_OK) return rc;
+  // the attention reads the rotated q the store leaves in q_out, contiguous [B, H, T, Dh]
+  const int64_t qo_strides[3] = {(int64_t)H * T * Dh, (int64_t)T * Dh, (int64_t)Dh};
+  we::AttnParams p;
+  AttnPlan pl;
+  rc = prepare_attn(q_out, qo_strides, kv, written, t_pos, out, out_strides, workspace, workspace_bytes, B, H, Hkv,
+                    T, Dh, L, dilation, scale, n_splits, q_tile, dtype, p, pl);
+  if (rc != WE_OK) return rc;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  // Everything is validated before the first launch; the kernels follow each other on the stream.
+  if (we::launch_rope_kv_store(sp, dtype, st) != hipSuccess) return WE_ERR_LAUNCH;
   if (we::launch_attn_ring(p, Dh, dtype, pl.variant == 1 ? 2 : 1, st) != hipSuccess) return WE_ERR_LAUNCH;
   if (pl.n_splits > 1 && we::launch_attn_combine(p, Dh, dtype, st) != hipSuccess) return WE_ERR_LAUNCH;
   return WE_OK;

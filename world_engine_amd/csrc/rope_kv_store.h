@@ -1,0 +1,164 @@
+// Per-item work of the fused RoPE + ring-slot K/V store kernel (rope_kv_store.hip, gfx950): one
+// item = 16 consecutive input elements of one (tensor, batch, head, token) row.
+#pragma once
+#include "we_common.h"
+#include "we_kernels.h"
+
+namespace we {
+
+struct Bf16Tag {
+  typedef uint16_t store_t;
+  static constexpr int kBytes = 2;
+  __device__ static float to_f32(uint16_t b) { return bf16_bits_to_f32(b); }
+  // v_cvt_pk_bf16_f32 (round-to-nearest-even) with c10::BFloat16's NaN (0x7FC0) patched in
+  __device__ static uint16_t from_f32(float f) {
+    const uint16_t r = __builtin_bit_cast(uint16_t, (__bf16)f);
+    return f != f ? (uint16_t)0x7fc0 : r;
+  }
+};
+struct F16Tag {
+  typedef uint16_t store_t;
+  static constexpr int kBytes = 2;
+  __device__ static float to_f32(uint16_t b) { return f16_bits_to_f32(b); }
+  __device__ static uint16_t from_f32(float f) { return f32_to_f16_bits(f); }
+};
+struct F32Tag {
+  typedef float store_t;
+  static constexpr int kBytes = 4;
+  __device__ static float to_f32(float b) { return b; }
+  __device__ static float from_f32(float f) { return f; }
+};
+
+// 16 elements of a row as raw storage.
+template <typename Tag>
+struct Chunk16 {
+  typename Tag::store_t e[16];
+};
+template <typename Tag>
+struct Chunk8 {
+  typename Tag::store_t e[8];
+};
+
+template <typename Tag>
+__device__ __forceinline__ void load16(Chunk16<Tag>& c, const void* p) {
+  constexpr int nvec = 16 * Tag::kBytes / 16;
+  const uint4* src = reinterpret_cast<const uint4*>(p);
+  uint4* dst = reinterpret_cast<uint4*>(c.e);
+#pragma unroll
+  for (int i = 0; i < nvec; ++i) dst[i] = src[i];
+}
+template <typename Tag>
+__device__ __forceinline__ void store16(void* p, const Chunk16<Tag>& c) {
+  constexpr int nvec = 16 * Tag::kBytes / 16;
+  uint4* dst = reinterpret_cast<uint4*>(p);
+  const uint4* src = reinterpret_cast<const uint4*>(c.e);
+#pragma unroll
+  for (int i = 0; i < nvec; ++i) dst[i] = src[i];
+}
+template <typename Tag>
+__device__ __forceinline__ void store8(void* p, const Chunk8<Tag>& c) {
+  constexpr int nvec = 8 * Tag::kBytes / 16;
+  uint4* dst = reinterpret_cast<uint4*>(p);
+  const uint4* src = reinterpret_cast<const uint4*>(c.e);
+#pragma unroll
+  for (int i = 0; i < nvec; ++i) dst[i] = src[i];
+}
+
+// Row of the cos / sin tables for token t of batch element b (src/model/attn.py:33-36): the
+// three position ids select one row of the flattened [frames, height, width] table.
+__device__ __forceinline__ int64_t rope_table_row(const StoreParams& p, int b, int t) {
+  int64_t pos = p.t_pos[b * p.pos_stride_b + t] * p.grid_hw + p.y_pos[b * p.pos_stride_b + t] * p.grid_w +
+                p.x_pos[b * p.pos_stride_b + t];
+  return pos < 0 ? 0 : (pos >= p.table_rows ? p.table_rows - 1 : pos);
+}
+
+// cos / sin of the 8 pairs of chunk `chunk` of a table row.
+__device__ __forceinline__ void load_cos_sin(const float* cos_row, const float* sin_row, int chunk, float (&c)[8],
+                                             float (&s)[8]) {
+  const float4* cp = reinterpret_cast<const float4*>(cos_row + chunk * 8);
+  const float4* sp = reinterpret_cast<const float4*>(sin_row + chunk * 8);
+  *reinterpret_cast<float4*>(c) = cp[0];
+  *reinterpret_cast<float4*>(c + 4) = cp[1];
+  *reinterpret_cast<float4*>(s) = sp[0];
+  *reinterpret_cast<float4*>(s + 4) = sp[1];
+}
+
+// Rotation of the 8 (even, odd) pairs of one 16-element chunk: lo gets x0*cos - x1*sin (elements
+// [8*chunk, 8*chunk+8) of the output row), hi gets x1*cos + x0*sin (the same range of the second
+// half; the reference concatenates the rotated halves, attn.py:38-40).  Every product and sum is
+// rounded separately, as eager fp32 tensor ops do: contraction into fused multiply-adds is
+// switched off for this function (plain operators; the pragma does not govern inlined intrinsics).
+template <typename Tag>
+__device__ __forceinline__ void rotate_values(const Chunk16<Tag>& in, const float (&c)[8], const float (&s)[8],
+                                              Chunk8<Tag>& lo, Chunk8<Tag>& hi) {
+#pragma clang fp contract(off)
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float x0 = Tag::to_f32(in.e[2 * i]);
+    const float x1 = Tag::to_f32(in.e[2 * i + 1]);
+    const float p0 = x0 * c[i], p1 = x1 * s[i], p2 = x1 * c[i], p3 = x0 * s[i];
+    const float y0 = p0 - p1;
+    const float y1 = p2 + p3;
+    lo.e[i] = Tag::from_f32(y0);
+    hi.e[i] = Tag::from_f32(y1);
+  }
+}
+template <typename Tag>
+__device__ __forceinline__ void rotate_chunk(const Chunk16<Tag>& in, const float* cos_row, const float* sin_row,
+                                             int chunk, Chunk8<Tag>& lo, Chunk8<Tag>& hi) {
+  float c[8], s[8];
+  load_cos_sin(cos_row, sin_row, chunk, c, s);
+  rotate_values<Tag>(in, c, s, lo, hi);
+}
+
+// Destination rows of a K/V item: tail always, ring slot on an unfrozen persisting frame.
+template <typename Tag>
+__device__ __forceinline__ void store_kv_rows(const StoreParams& p, int which, int b, int h, int t, int chunk,
+                                              const SlotInfo& si, bool rotated, const Chunk16<Tag>& in,
+                                              const Chunk8<Tag>& lo, const Chunk8<Tag>& hi) {
+  typedef typename Tag::store_t st_t;
+  const int64_t cap = p.L + p.T;
+  const int plane = which - 1;
+  st_t* plane_base = (st_t*)p.kv + (((int64_t)plane * p.B + b) * p.Hkv + h) * cap * p.Dh;
+  const bool to_ring = (!p.frozen) && si.write_step;
+  const int64_t tail_row = p.L + t;
+  const int64_t ring_row = (int64_t)si.slot * p.T + t;
+  st_t* d0 = plane_base + tail_row * p.Dh;
+  st_t* d1 = plane_base + ring_row * p.Dh;
+  if (rotated) {
+    store8<Tag>(d0 + chunk * 8, lo);
+    store8<Tag>(d0 + (p.Dh >> 1) + chunk * 8, hi);
+    if (to_ring) {
+      store8<Tag>(d1 + chunk * 8, lo);
+      store8<Tag>(d1 + (p.Dh >> 1) + chunk * 8, hi);
+    }
+  } else {
+    store16<Tag>(d0 + chunk * 16, in);
+    if (to_ring) store16<Tag>(d1 + chunk * 16, in);
+  }
+  // written[dst] = True for the rows the unfrozen write went to (kv_cache.py:149-151).
+  if (!p.frozen && which == 1 && b == 0 && h == 0 && chunk == 0) p.written[to_ring ? ring_row : tail_row] = 1;
+}
+
+// One K (which = 1) or V (which = 2) item: rotate K, copy V; write the tail row always and the
+// ring-slot row when this is an unfrozen persisting frame; mark `written`
+// (src/model/kv_cache.py:138,147-151).
+template <typename Tag>
+__device__ __forceinline__ void store_kv_item(const StoreParams& p, int which, int b, int h, int t, int chunk,
+                                              const SlotInfo& si) {
+  typedef typename Tag::store_t st_t;
+  const st_t* src = which == 1 ? (const st_t*)p.k + b * p.ks_b + h * p.ks_h + t * p.ks_t
+                               : (const st_t*)p.v + b * p.vs_b + h * p.vs_h + t * p.vs_t;
+  Chunk16<Tag> in;
+  load16<Tag>(in, src + chunk * 16);
+  const bool rotate = which == 1 && p.cos_t != nullptr;
+  Chunk8<Tag> lo, hi;
+  if (rotate) {
+    const int64_t pos = rope_table_row(p, b, t);
+    const int half = p.Dh >> 1;
+    rotate_chunk<Tag>(in, p.cos_t + pos * half, p.sin_t + pos * half, chunk, lo, hi);
+  }
+  store_kv_rows<Tag>(p, which, b, h, t, chunk, si, rotate, in, lo, hi);
+}
+
+}  // namespace we

@@ -199,6 +199,60 @@ def attn_ring(q: Tensor, kv: Tensor, written: Tensor, t_pos: Tensor, L: int, dil
     return out
 
 
+def rope_kv_attn(q: Tensor, k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor], cos_table: Tensor,
+                 sin_table: Tensor, grid_h: int, grid_w: int, kv: Tensor, written: Tensor, L: int,
+                 dilation: int, is_frozen: bool, scale: Optional[float] = None, n_splits: int = 0,
+                 q_tile: int = 0, out: Optional[Tensor] = None, workspace: Optional[Tensor] = None,
+                 token_major_out: bool = True):
+    """``rope_kv_store`` followed by ``attn_ring`` in one library call (``we_rope_kv_attn_fwd``):
+    the per-layer sequence of the reference from ``q, k = rope(q), rope(k)`` to the
+    ``flex_attention`` call (``src/model/attn.py:110-116``), validated as a whole before the first
+    launch.  Returns ``(out, q_rot)``; results are those of the two separate calls, bit for bit."""
+    dev = _need_device(q, k, v, kv, written, cos_table, sin_table, pos_ids["t_pos"])
+    if k.dim() != 4 or k.shape != v.shape:
+        raise RuntimeError("k and v must both be [B, Hkv, T, Dh]")
+    B, Hkv, T, Dh = k.shape
+    if q.dim() != 4 or q.shape[0] != B or q.shape[2] != T or q.shape[3] != Dh:
+        raise RuntimeError("q must be [B, H, T, Dh] matching k")
+    H = q.shape[1]
+    if k.dtype != kv.dtype or v.dtype != kv.dtype or q.dtype != kv.dtype:
+        raise RuntimeError("q/k/v must have the cache's element type")
+    if kv.dim() != 5 or tuple(kv.shape) != (2, B, Hkv, L + T, Dh) or not kv.is_contiguous():
+        raise RuntimeError("kv must be a contiguous [2, B, Hkv, L+T, Dh] buffer; "
+                           "KV cache expects exactly one frame per upsert")
+    if written.dtype != torch.bool or written.numel() != L + T or not written.is_contiguous():
+        raise RuntimeError("written must be a contiguous bool [L+T] tensor")
+    if (cos_table.dtype != torch.float32 or sin_table.dtype != torch.float32
+            or cos_table.shape != sin_table.shape or cos_table.dim() != 2 or cos_table.shape[1] != Dh // 2
+            or not cos_table.is_contiguous() or not sin_table.is_contiguous()):
+        raise RuntimeError("cos/sin tables must be contiguous fp32 [rows, Dh/2]")
+    t_pos, y_pos, x_pos, ps = _pos_triplet(pos_ids, B, T, True)
+    scale = 1.0 / math.sqrt(Dh) if scale is None else float(scale)
+    lib = _capi.lib()
+    ws_bytes = int(lib.we_attn_workspace_bytes(B, H, Hkv, T, Dh, L, n_splits, q_tile))
+    if ws_bytes and (workspace is None or workspace.numel() * workspace.element_size() < ws_bytes):
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    q_rot = torch.empty((B, H, T, Dh), dtype=q.dtype, device=dev)
+    if out is None:
+        if token_major_out:
+            out = torch.empty((B, T, H, Dh), dtype=q.dtype, device=dev).transpose(1, 2)
+        else:
+            out = torch.empty((B, H, T, Dh), dtype=q.dtype, device=dev)
+    elif tuple(out.shape) != (B, H, T, Dh) or out.dtype != q.dtype or out.device != dev:
+        raise RuntimeError("out must be [B, H, T, Dh] of q's element type on q's device")
+    code = lib.we_rope_kv_attn_fwd(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), _bhtd_strides(q, "q"), _bhtd_strides(k, "k"), _bhtd_strides(v, "v"),
+        q_rot.data_ptr(), cos_table.data_ptr(), sin_table.data_ptr(), cos_table.shape[0],
+        t_pos.data_ptr(), y_pos.data_ptr(), x_pos.data_ptr(), ps, grid_h, grid_w, kv.data_ptr(), written.data_ptr(),
+        out.data_ptr(), _bhtd_strides(out, "out"),
+        workspace.data_ptr() if ws_bytes else None,
+        workspace.numel() * workspace.element_size() if ws_bytes else 0,
+        B, H, Hkv, T, Dh, L, dilation, int(bool(is_frozen)), scale, n_splits, q_tile, _dtype_code(kv),
+        _stream_ptr(dev))
+    _capi.check(code, "we_rope_kv_attn_fwd")
+    return out, q_rot
+
+
 # --------------------------------------------------------------------------------------------
 # torch.library registration: opaque ops that survive torch.compile(fullgraph=True), the way the
 # reference wraps its one native kernel (src/quantize.py:17-42).
