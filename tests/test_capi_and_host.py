@@ -162,3 +162,23 @@ def test_custom_ops_registered_with_fake_kernels():
     tab = torch.empty(64, 32, device="meta")
     qr = torch.ops.world_engine_amd.rope_kv_store(q, q, q, t, t, t, tab, tab, 8, 8, kv, written, 128, 1, False)
     assert qr.shape == q.shape
+    y = torch.ops.world_engine_amd.rope_kv_attn(q, q, q, t, t, t, tab, tab, 8, 8, kv, written, 128, 1, False, 0.125)
+    assert y.shape == (1, 4, 64, 64) and y.transpose(1, 2).is_contiguous()
+
+
+def test_one_call_entry_point_validates_both_halves():
+    lib = _capi.lib()
+    s3 = _capi.i64x3(8, 8, 8)
+    fake = ctypes.c_void_p(4096)     # never dereferenced: validation fails first
+    args = lambda **kw: [kw.get("q", fake), fake, fake, s3, s3, s3, kw.get("q_out", fake), kw.get("cos", fake), fake, 10,
+                         fake, fake, fake, 64, 8, 8, fake, fake, kw.get("out", fake), s3, None, 0,
+                         1, 1, 1, 64, kw.get("Dh", 64), kw.get("L", 64), 1, 0, 0.1, kw.get("n_splits", 1), 0,
+                         kw.get("dtype", 0), None]
+    assert lib.we_rope_kv_attn_fwd(*args(q=None)) == -1
+    assert lib.we_rope_kv_attn_fwd(*args(q_out=None)) == -1
+    assert lib.we_rope_kv_attn_fwd(*args(cos=None)) == -1
+    assert lib.we_rope_kv_attn_fwd(*args(out=None)) == -1            # attention half
+    assert lib.we_rope_kv_attn_fwd(*args(L=100)) == -2
+    assert lib.we_rope_kv_attn_fwd(*args(Dh=96)) == -3               # store accepts it, attention does not
+    assert lib.we_rope_kv_attn_fwd(*args(dtype=2)) == -3             # fp32: store only
+    assert lib.we_rope_kv_attn_fwd(*args(n_splits=2)) == -5          # splits without workspace

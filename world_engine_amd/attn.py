@@ -141,9 +141,13 @@ class RingAttn(nn.Module):
         q = F.rms_norm(q, (self.d_head,))
         k = F.rms_norm(k, (self.d_head,))
 
-        # RoPE(q), RoPE(k), cache write: one launch.  Attention over the ring: one or two.
-        q, k_all, v_all, ring = kv_cache.rope_upsert(q, k, v, pos_ids, self.rope, self.layer_idx)
-        y = ring_attention(q, k_all, v_all, ring, enable_gqa=self.enable_gqa)
+        # RoPE(q), RoPE(k), cache write (one launch) and attention over the ring (one or two), all
+        # behind one library call; a cache without it gets the reference's sequence of calls
+        if hasattr(kv_cache, "rope_upsert_attend"):
+            y = kv_cache.rope_upsert_attend(q, k, v, pos_ids, self.rope, self.layer_idx)
+        else:
+            q, k_all, v_all, ring = kv_cache.rope_upsert(q, k, v, pos_ids, self.rope, self.layer_idx)
+            y = ring_attention(q, k_all, v_all, ring, enable_gqa=self.enable_gqa)
 
         if self.gated_attn:
             gates = torch.sigmoid(self.gate_proj(x[..., : self.n_heads]))

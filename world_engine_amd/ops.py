@@ -282,3 +282,19 @@ def attn_ring_op(q: Tensor, kv: Tensor, written: Tensor, t_pos: Tensor, L: int, 
 def _attn_ring_fake(q, kv, written, t_pos, L, dilation, scale):
     B, H, T, Dh = q.shape
     return q.new_empty((B, T, H, Dh)).transpose(1, 2)
+
+
+@torch.library.custom_op("world_engine_amd::rope_kv_attn", mutates_args=("kv", "written"))
+def rope_kv_attn_op(q: Tensor, k: Tensor, v: Tensor, t_pos: Tensor, y_pos: Tensor, x_pos: Tensor,
+                    cos_table: Tensor, sin_table: Tensor, grid_h: int, grid_w: int,
+                    kv: Tensor, written: Tensor, L: int, dilation: int, is_frozen: bool, scale: float) -> Tensor:
+    pos = {"t_pos": t_pos, "y_pos": y_pos, "x_pos": x_pos}
+    return rope_kv_attn(q, k, v, pos, cos_table, sin_table, grid_h, grid_w, kv, written, L, dilation,
+                        is_frozen, scale)[0]
+
+
+@rope_kv_attn_op.register_fake
+def _rope_kv_attn_fake(q, k, v, t_pos, y_pos, x_pos, cos_table, sin_table, grid_h, grid_w, kv, written, L,
+                       dilation, is_frozen, scale):
+    B, H, T, Dh = q.shape
+    return q.new_empty((B, T, H, Dh)).transpose(1, 2)
