@@ -46,7 +46,8 @@ def test_validation_codes_without_gpu():
     # unsupported head dim / frame length / dtype / slot count
     assert lib.we_attn_ring_fwd(fake, s3, fake, fake, fake, fake, s3, None, 0, 1, 1, 1, 64, 96, 64, 1, 0.1, 1, 0, 0, None) == -3
     assert lib.we_attn_ring_fwd(fake, s3, fake, fake, fake, fake, s3, None, 0, 1, 1, 1, 48, 64, 96, 1, 0.1, 1, 0, 0, None) == -3
-    assert lib.we_attn_ring_fwd(fake, s3, fake, fake, fake, fake, s3, None, 0, 1, 1, 1, 64, 64, 64, 1, 0.1, 1, 0, 2, None) == -3
+    assert lib.we_attn_ring_fwd(fake, s3, fake, fake, fake, fake, s3, None, 0, 1, 1, 1, 64, 64, 64, 1, 0.1, 1, 0, 3, None) == -3
+    assert lib.we_attn_ring_fwd(fake, s3, fake, fake, fake, fake, s3, None, 0, 1, 1, 1, 64, 64, 64, 1, 0.1, 2, 0, 2, None) == -3   # fp32: no splits
     assert lib.we_attn_ring_fwd(fake, s3, fake, fake, fake, fake, s3, None, 0, 1, 1, 1, 64, 64, 64 * 257, 1, 0.1, 1, 0, 0, None) == -3
     # misaligned pointer / stride
     assert lib.we_attn_ring_fwd(ctypes.c_void_p(4100), s3, fake, fake, fake, fake, s3, None, 0, 1, 1, 1, 64, 64, 64, 1, 0.1, 1, 0, 0, None) == -4
@@ -180,5 +181,6 @@ def test_one_call_entry_point_validates_both_halves():
     assert lib.we_rope_kv_attn_fwd(*args(out=None)) == -1            # attention half
     assert lib.we_rope_kv_attn_fwd(*args(L=100)) == -2
     assert lib.we_rope_kv_attn_fwd(*args(Dh=96)) == -3               # store accepts it, attention does not
-    assert lib.we_rope_kv_attn_fwd(*args(dtype=2)) == -3             # fp32: store only
+    assert lib.we_rope_kv_attn_fwd(*args(dtype=2, n_splits=2)) == -3 # fp32 runs the one-pass kernel only
+    assert lib.we_rope_kv_attn_fwd(*args(dtype=3)) == -3
     assert lib.we_rope_kv_attn_fwd(*args(n_splits=2)) == -5          # splits without workspace

@@ -116,6 +116,35 @@ def test_attention_cfg0_shapes_bf16(gpu_device):
     _say(f"cfg0 shapes: worst max-abs {worst[0]:.2e} mean-abs {worst[1]:.2e}")
 
 
+def test_attention_cfg0_fp32(gpu_device):
+    """BASELINE config 0 as stated (fp32, B=1, H=8, Dh=64, 64-token frames, 4 slots, 8 steps, the
+    ring wraps twice) through the fp32 kernel: fp32 arithmetic throughout, so the bar is 1e-5."""
+    p = Pair(gpu_device, torch.float32, B=1, H=8, Hkv=8, T=64, Dh=64, n_slots=4, cfg_id=0)
+    p.set_frozen(False)
+    for t in range(8):
+        q, k, v, pos = p.inputs(t)
+        (q_o, k_all, v_all, mask), (q_h, ring) = p.store(q, k, v, pos)
+        out = p.attend(q_h, ring)
+        p.assert_state_equal(what=f"t={t}")
+        ref = ro.attention_reference_path(q_o, k_all, v_all, mask)     # fp32 inputs: the reference's own flow
+        diff = (out.cpu() - ref).abs()
+        assert diff.max().item() <= 1e-5, f"t={t}: max-abs {diff.max().item():.2e}"
+        assert out.transpose(1, 2).is_contiguous()
+
+
+@pytest.mark.parametrize("Dh,hkv,T", [(128, 2, 128), (64, 4, 192)])
+def test_attention_fp32_other_shapes(gpu_device, Dh, hkv, T):
+    """fp32 kernel with grouped heads, both head dims, several query tiles and a dilated ring."""
+    p = Pair(gpu_device, torch.float32, B=2, H=4, Hkv=hkv, T=T, Dh=Dh, n_slots=4, d=2, cfg_id=41)
+    for t in range(7):
+        p.set_frozen(t % 3 == 2)
+        q, k, v, pos = p.inputs(t)
+        (q_o, k_all, v_all, mask), (q_h, ring) = p.store(q, k, v, pos)
+        out = p.attend(q_h, ring)
+        ref = ro.attention_fp32(q_o, k_all, v_all, mask)
+        assert (out.cpu() - ref).abs().max().item() <= 1e-5, f"t={t}"
+
+
 def test_attention_cfg1_all_32_steps(gpu_device):
     """BASELINE config 1: B=1,H=16,Dh=128,T=256, 16 slots, 32 steps (warm-up + steady wrap)."""
     p = Pair(gpu_device, torch.bfloat16, B=1, H=16, Hkv=16, T=256, Dh=128, n_slots=16, cfg_id=1)
@@ -341,7 +370,8 @@ def test_bad_inputs_raise(gpu_device):
     with pytest.raises(RuntimeError, match="not covered"):
         ops.attn_ring(torch.zeros(1, 1, 64, 32, dtype=torch.bfloat16, device=dev), layer.kv, layer.written,
                       torch.zeros(1, 64, dtype=torch.long, device=dev), 64, 1)
+    # fp32 caches run the one-pass kernel: asking for a context split is refused
     with pytest.raises(RuntimeError, match="not covered"):
         lay32 = wea.LayerKVCache(1, 1, 128, 64, torch.float32, 64).to(dev)
         ops.attn_ring(torch.zeros(1, 1, 64, 64, dtype=torch.float32, device=dev), lay32.kv, lay32.written,
-                      torch.zeros(1, 64, dtype=torch.long, device=dev), 128, 1)
+                      torch.zeros(1, 64, dtype=torch.long, device=dev), 128, 1, n_splits=2)

@@ -7,7 +7,7 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
-SOURCES = ["rope_kv_store.hip", "attn_ring.hip", "attn_combine.hip", "capi.hip"]
+SOURCES = ["rope_kv_store.hip", "attn_ring.hip", "attn_ring_f32.hip", "attn_combine.hip", "capi.hip"]
 OUT = os.path.join(HERE, "libwe_attn.so")
 
 HIPCC_FLAGS = [

@@ -129,12 +129,17 @@ int prepare_attn(const void* q, const int64_t* q_strides, const void* kv, const 
   if (!q || !q_strides || !kv || !written || !t_pos || !out || !out_strides) return WE_ERR_NULL_POINTER;
   int rc = ring_shape_ok(B, H, Hkv, T, Dh, L, dilation);
   if (rc != WE_OK) return rc;
-  if (dtype != WE_DTYPE_BF16 && dtype != WE_DTYPE_F16) return WE_ERR_UNSUPPORTED;
+  if (dtype != WE_DTYPE_BF16 && dtype != WE_DTYPE_F16 && dtype != WE_DTYPE_F32) return WE_ERR_UNSUPPORTED;
   if (Dh != 64 && Dh != 128) return WE_ERR_UNSUPPORTED;
   if (T % 64 != 0 || L / T > WE_MAX_SLOTS) return WE_ERR_UNSUPPORTED;
   if ((uint64_t)(L + T) * (uint64_t)Dh * 2u >= (1ull << 32)) return WE_ERR_UNSUPPORTED;  // 32-bit tile offsets
   if (!(scale > 0.f) || n_splits < 0 || n_splits > 64) return WE_ERR_BAD_SHAPE;
   if (variant_of(q_tile) < 0) return WE_ERR_UNSUPPORTED;
+  if (dtype == WE_DTYPE_F32) {
+    // fp32 caches take the plain one-pass kernel: no context splitting, no tile choice
+    if (n_splits > 1 || H > 65535 || B > 65535) return WE_ERR_UNSUPPORTED;
+    n_splits = 1;
+  }
   if (!aligned16(q) || !aligned16(kv) || !aligned16(out) || !strides_ok(q_strides, dtype) ||
       !strides_ok(out_strides, dtype))
     return WE_ERR_ALIGNMENT;
@@ -165,6 +170,13 @@ int prepare_attn(const void* q, const int64_t* q_strides, const void* kv, const 
 
   if ((p.unit_splits + 7) / 8 > 65535 || p.group > 65535 || (int64_t)B * H - (int64_t)pl.units_whole * p.group > 65535)
     return WE_ERR_UNSUPPORTED;  // grid y / z limits of the two launches
+  return WE_OK;
+}
+
+int launch_attn(const we::AttnParams& p, const AttnPlan& pl, int Dh, int dtype, hipStream_t st) {
+  if (dtype == WE_DTYPE_F32) return we::launch_attn_ring_f32(p, Dh, st) == hipSuccess ? WE_OK : WE_ERR_LAUNCH;
+  if (we::launch_attn_ring(p, Dh, dtype, pl.variant == 1 ? 2 : 1, st) != hipSuccess) return WE_ERR_LAUNCH;
+  if (pl.n_splits > 1 && we::launch_attn_combine(p, Dh, dtype, st) != hipSuccess) return WE_ERR_LAUNCH;
   return WE_OK;
 }
 
@@ -258,9 +270,7 @@ int we_attn_ring_fwd(const void* q, const int64_t q_strides[3], const void* kv, 
                               Hkv, T, Dh, L, dilation, scale, n_splits, q_tile, dtype, p, pl);
   if (rc != WE_OK) return rc;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (we::launch_attn_ring(p, Dh, dtype, pl.variant == 1 ? 2 : 1, st) != hipSuccess) return WE_ERR_LAUNCH;
-  if (pl.n_splits > 1 && we::launch_attn_combine(p, Dh, dtype, st) != hipSuccess) return WE_ERR_LAUNCH;
-  return WE_OK;
+  return launch_attn(p, pl, Dh, dtype, st);
 }
 
 int we_rope_kv_attn_fwd(const void* q, const void* k, const void* v, const int64_t q_strides[3],
@@ -288,9 +298,7 @@ int we_rope_kv_attn_fwd(const void* q, const void* k, const void* v, const int64
   hipStream_t st = static_cast<hipStream_t>(stream);
   // Everything is validated before the first launch; the kernels follow each other on the stream.
   if (we::launch_rope_kv_store(sp, dtype, st) != hipSuccess) return WE_ERR_LAUNCH;
-  if (we::launch_attn_ring(p, Dh, dtype, pl.variant == 1 ? 2 : 1, st) != hipSuccess) return WE_ERR_LAUNCH;
-  if (pl.n_splits > 1 && we::launch_attn_combine(p, Dh, dtype, st) != hipSuccess) return WE_ERR_LAUNCH;
-  return WE_OK;
+  return launch_attn(p, pl, Dh, dtype, st);
 }
 
 }  // extern "C"

@@ -57,6 +57,8 @@ hipError_t launch_rope_kv_store(const StoreParams& p, int dtype, hipStream_t str
 
 // main kernel: ksplit = 2 -> 128 queries per workgroup, 1 -> 256
 hipError_t launch_attn_ring(const AttnParams& p, int Dh, int dtype, int ksplit, hipStream_t stream);
+// fp32 caches: plain vector-ALU kernel, one pass, no context splitting
+hipError_t launch_attn_ring_f32(const AttnParams& p, int Dh, hipStream_t stream);
 hipError_t launch_attn_combine(const AttnParams& p, int Dh, int dtype, hipStream_t stream);
 
 }  // namespace we
