@@ -141,7 +141,8 @@ size_t we_attn_workspace_bytes(int32_t B, int32_t H, int32_t Hkv, int32_t T, int
  *
  * Requirements: dtype bf16 or f16 (MFMA kernel) or f32 (plain one-pass kernel on the vector
  * ALUs, fp32 arithmetic throughout, n_splits 0 or 1, q_tile ignored); Dh in {64, 128};
- * T % 64 == 0; L/T <= WE_MAX_SLOTS; H % Hkv == 0; pointers and row starts 16-byte aligned.
+ * any T (frames that are not a multiple of the 64-key tile cost one masked tile per slot);
+ * L/T <= WE_MAX_SLOTS; H % Hkv == 0; pointers and row starts 16-byte aligned.
  */
 int we_attn_ring_fwd(const void* q, const int64_t q_strides[3],
                      const void* kv, const uint8_t* written, const int64_t* t_pos,

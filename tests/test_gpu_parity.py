@@ -173,6 +173,27 @@ def test_attention_dtypes_head_dims_and_ragged_tiles(gpu_device, dtype, Dh, T):
         _run_and_check(p, 5, **kw)
 
 
+@pytest.mark.parametrize("T,Dh,kw", [(80, 128, {}), (96, 64, {}), (40, 128, {}), (200, 128, {"n_splits": 3}),
+                                     (330, 64, {"q_tile": 256, "n_splits": 2}), (24, 128, {"n_splits": 1}),
+                                     (136, 128, {"q_tile": 256})])
+def test_attention_frame_lengths_off_the_tile_grid(gpu_device, T, Dh, kw):
+    """Frame lengths that are not multiples of the 64-key tile (or of 32, or below one block):
+    the last tile of every slot is short, its missing keys must not count and the rows behind it
+    (the next slot's frame, or the end of the buffer for the tail) must not be read as keys."""
+    _say(f"ragged T={T} Dh={Dh} {kw}")
+    p = Pair(gpu_device, torch.bfloat16, B=2, H=2, Hkv=1, T=T, Dh=Dh, n_slots=3, cfg_id=51)
+    _run_and_check(p, 8, frozen_subs=1, **kw)
+
+
+def test_attention_fp32_ragged_frame(gpu_device):
+    p = Pair(gpu_device, torch.float32, B=1, H=2, Hkv=2, T=72, Dh=64, n_slots=3, cfg_id=52)
+    for t in range(7):
+        p.set_frozen(False)
+        q, k, v, pos = p.inputs(t)
+        (q_o, k_all, v_all, mask), (q_h, ring) = p.store(q, k, v, pos)
+        assert (p.attend(q_h, ring).cpu() - ro.attention_fp32(q_o, k_all, v_all, mask)).abs().max().item() <= 1e-5
+
+
 def test_attention_partial_round_tail_split(gpu_device):
     """320 workgroups = one full round of 256 CUs plus a quarter round: the library splits the
     context of the last 32 heads only (mixed direct-output and workspace rows in one call)."""

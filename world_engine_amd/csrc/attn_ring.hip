@@ -100,8 +100,11 @@ __device__ __forceinline__ u32x2_t lds_read_tr(const unsigned char* smem, uint32
   return __builtin_bit_cast(u32x2_t, v);
 }
 
-template <typename M, int DH, int KSPLIT>
-__global__ void __launch_bounds__(512, 2) attn_ring_kernel(AttnParams p) {
+// RAGGED: the frame length is not a multiple of the 64-key tile (separate instantiation: the
+// masking of the short tiles costs registers the common case cannot spare).
+template <typename M, int DH, int KSPLIT, bool RAGGED>
+__global__ void __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_per_eu(2, 2)))
+attn_ring_kernel(AttnParams p) {
   typedef typename M::frag_t frag_t;
   typedef RingLds<DH> L;
   constexpr int KS = DH / 16;               // contraction steps of K Q^T
@@ -184,7 +187,10 @@ __global__ void __launch_bounds__(512, 2) attn_ring_kernel(AttnParams p) {
     if (__builtin_expect(i < 64, 1)) return __builtin_amdgcn_readlane(vis0, i);
     return __builtin_amdgcn_readfirstlane(vis[i]);
   };
-  const int tps = p.T / BN;  // tiles per slot
+  // tiles per slot; the last one of a slot holds t_last of its 64 keys when T % 64 != 0
+  const int tps = (p.T + BN - 1) / BN;
+  const int t_last = p.T - (tps - 1) * BN;
+  constexpr bool ragged = RAGGED;
   const int nt = nvis * tps;
   int t_begin = 0, t_end = nt;
   if (nsp > 1) {  // nt <= 257 * T / 64 and nsp <= 64: the products fit 32 bits
@@ -226,21 +232,47 @@ __global__ void __launch_bounds__(512, 2) attn_ring_kernel(AttnParams p) {
       }
     }
   };
-  // byte offset of a tile inside its (batch, kv head) plane; fits 32 bits (checked on the host)
+  // byte offset of a tile inside its (batch, kv head) plane; fits 32 bits (checked on the host).
+  // Bit 0 (row starts are multiples of 128 bytes) marks the short last tile of a slot.
   auto tile_off = [&](const TileWalk& w) __attribute__((always_inline)) {
-    return (uint32_t)(vis_at(w.sidx) * p.T + w.sub * BN) * (uint32_t)ROW_B;
+    const uint32_t o = (uint32_t)(vis_at(w.sidx) * p.T + w.sub * BN) * (uint32_t)ROW_B;
+    return (ragged && w.sub == tps - 1) ? (o | 1u) : o;
   };
   const uint64_t kplane = uniform64(kbase), vplane = uniform64(vbase);
+  // A short tile must not read rows of the next slot (or past the end of the buffer): its rows
+  // beyond t_last repeat row t_last - 1; their keys are masked out of the softmax further down.
+  auto clamp_rows = [&](uint32_t voff, int i) __attribute__((always_inline)) {
+    const int row = (wave + i * 8) * RPI + lane / CPR;
+    return row < t_last ? voff : voff - (uint32_t)(row - (t_last - 1)) * ROW_B;
+  };
   auto dma_k = [&](uint32_t off, int slot) __attribute__((always_inline)) {
+    const bool cut = (off & 1u) != 0u;
+    off &= ~1u;
 #pragma unroll
     for (int i = 0; i < NDMA; ++i)
-      dma16(kplane, kvoff[i] + off, __builtin_amdgcn_readfirstlane(lds0 + slot * TILE_B + (wave + i * 8) * 1024));
+      dma16(kplane, (cut ? clamp_rows(kvoff[i], i) : kvoff[i]) + off,
+            __builtin_amdgcn_readfirstlane(lds0 + slot * TILE_B + (wave + i * 8) * 1024));
   };
   auto dma_v = [&](uint32_t off, int slot) __attribute__((always_inline)) {
+    const bool cut = (off & 1u) != 0u;
+    off &= ~1u;
 #pragma unroll
     for (int i = 0; i < NDMA; ++i)
-      dma16(vplane, vvoff[i] + off,
+      dma16(vplane, (cut ? clamp_rows(vvoff[i], i) : vvoff[i]) + off,
             __builtin_amdgcn_readfirstlane(lds0 + L::V_OFF + slot * TILE_B + (wave + i * 8) * 1024));
+  };
+  // keys of 32-key block blk of the tile at position sub of its slot that exist (0 .. 32)
+  auto block_keys = [&](int sub, int blk) __attribute__((always_inline)) {
+    if (!RAGGED) return 32;
+    const int n = ((ragged && sub == tps - 1) ? t_last : BN) - 32 * blk;
+    return n < 0 ? 0 : (n > 32 ? 32 : n);
+  };
+  // logits of keys that do not exist become -inf (register i of a lane is key row
+  // (i / 4) * 8 + 4 * hh + i % 4 of the block)
+  auto mask_keys = [&](f32x16_t& sv, int nkeys) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      if ((i / 4) * 8 + 4 * hh + (i % 4) >= nkeys) sv[i] = -INFINITY;
   };
 
   // ---- fragment read addresses (byte offsets into smem) ----
@@ -339,7 +371,10 @@ __global__ void __launch_bounds__(512, 2) attn_ring_kernel(AttnParams p) {
     for (int ks = 0; ks < KS; ++ks) read_k(koff_c, ks);
     read_v(voff_c, 0);
   };
-  auto step = [&](auto koff_c, auto voff_c, auto nkoff_c, auto nvoff_c, bool live, auto&& mid) __attribute__((always_inline)) {
+  // nkeys: keys that exist in the block whose logits this step computes (32 = all, 0 = the block
+  // lies past the end of the split)
+  auto step = [&](auto koff_c, auto voff_c, auto nkoff_c, auto nvoff_c, int nkeys, auto&& mid) __attribute__((always_inline)) {
+    const bool live = nkeys > 0;
     if (pending) {
 #pragma unroll
       for (int db = 0; db < DB; ++db)
@@ -440,6 +475,7 @@ __global__ void __launch_bounds__(512, 2) attn_ring_kernel(AttnParams p) {
     l_run += rs;
     p_prev[0] = p_cur[0];
     p_prev[1] = p_cur[1];
+    if (RAGGED && nkeys > 0 && nkeys < 32) mask_keys(s_next, nkeys);  // short last tile of a slot
     s_cur = s_next;
   };
 
@@ -458,6 +494,7 @@ __global__ void __launch_bounds__(512, 2) attn_ring_kernel(AttnParams p) {
     constexpr int KA = KSPLIT == 1 ? 3 : 4;
     // The V stream trails the K stream by KA - 2 tiles, so it reuses the K stream's offsets.
     TileWalk kw = walk_init();
+    int csub = kw.sub;  // position in its slot of the tile whose logits are computed next
     uint32_t off1, off2;  // offsets of the last and the last-but-one tile the K stream visited
     // Q was requested before the slot flags and loads return in order, so it is here; stating a
     // use now keeps the wait for it from landing behind the tile DMAs issued next.
@@ -500,7 +537,10 @@ __global__ void __launch_bounds__(512, 2) attn_ring_kernel(AttnParams p) {
         const frag_t a = *reinterpret_cast<const frag_t*>(smem + (k_rd ^ (ks << 5)));
         s_cur = M::mma(a, qf[ks], s_cur);
       }
-      m_ref = M::round_up(block_max(s_cur));
+      const int nk0 = block_keys(csub, hb);
+      if (RAGGED && nk0 < 32) mask_keys(s_cur, nk0);
+      const float mx0 = block_max(s_cur);
+      m_ref = mx0 > -INFINITY ? M::round_up(mx0) : 0.f;  // (a block of the first tile may be empty)
       set_shift();
 #pragma unroll
       for (int i = 0; i < 16; ++i) s_cur[i] -= m_ref;
@@ -523,18 +563,23 @@ __global__ void __launch_bounds__(512, 2) attn_ring_kernel(AttnParams p) {
         off1 = o;
       };
       auto nothing = [&]() __attribute__((always_inline)) {};
+      // csub is tile j's position in its slot; nsub tile j+1's
+      const int nsub = csub + 1 == tps ? 0 : csub + 1;
       if (KSPLIT == 1) {
         // block (j, 0) -> probabilities; logits of (j, 1); product of (j-1, 1)
         step(IntC<JM * TILE_B + KB_B>(), IntC<((JM + 3) % NST) * TILE_B + KB_B>(),
-             IntC<((JM + 1) % NST) * TILE_B>(), IntC<JM * TILE_B>(), true, issue_dma);
+             IntC<((JM + 1) % NST) * TILE_B>(), IntC<JM * TILE_B>(), block_keys(csub, 1), issue_dma);
         // block (j, 1) -> probabilities; logits of (j+1, 0); product of (j, 0)
         step(IntC<((JM + 1) % NST) * TILE_B>(), IntC<JM * TILE_B>(),
-             IntC<((JM + 1) % NST) * TILE_B + KB_B>(), IntC<JM * TILE_B + KB_B>(), j + 1 < ntile, nothing);
+             IntC<((JM + 1) % NST) * TILE_B + KB_B>(), IntC<JM * TILE_B + KB_B>(),
+             j + 1 < ntile ? block_keys(nsub, 0) : 0, nothing);
       } else {
         // block (j, hb) -> probabilities; logits of (j+1, hb); product of (j-1, hb)
         step(IntC<((JM + 1) % NST) * TILE_B>(), IntC<((JM + 3) % NST) * TILE_B>(),
-             IntC<((JM + 2) % NST) * TILE_B>(), IntC<JM * TILE_B>(), j + 1 < ntile, issue_dma);
+             IntC<((JM + 2) % NST) * TILE_B>(), IntC<JM * TILE_B>(),
+             j + 1 < ntile ? block_keys(nsub, __builtin_amdgcn_readfirstlane(hb)) : 0, issue_dma);
       }
+      csub = nsub;
       dma_wait<2 * NDMA>();  // all but this iteration's two tiles have landed (this wavefront's part)
       __syncthreads();
     };
@@ -651,20 +696,24 @@ __global__ void __launch_bounds__(512, 2) attn_ring_kernel(AttnParams p) {
   }
 }
 
-template <typename M, int DH, int KSPLIT>
-static hipError_t launch_ring_t(const AttnParams& p, hipStream_t stream) {
+template <typename M, int DH, int KSPLIT, bool RAGGED>
+static hipError_t launch_ring_r(const AttnParams& p, hipStream_t stream) {
   static bool configured = false;
   const int lds = RingLds<DH>::kBytes;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_ring_kernel<M, DH, KSPLIT>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_ring_kernel<M, DH, KSPLIT, RAGGED>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
     configured = true;
   }
   const int rounds = (p.unit_splits + 7) / 8;
   const dim3 grid((unsigned)(8 * p.q_tiles), (unsigned)p.group, (unsigned)rounds);
-  hipLaunchKernelGGL((attn_ring_kernel<M, DH, KSPLIT>), grid, dim3(512), lds, stream, p);
+  hipLaunchKernelGGL((attn_ring_kernel<M, DH, KSPLIT, RAGGED>), grid, dim3(512), lds, stream, p);
   return hipGetLastError();
+}
+template <typename M, int DH, int KSPLIT>
+static hipError_t launch_ring_t(const AttnParams& p, hipStream_t stream) {
+  return p.T % BN == 0 ? launch_ring_r<M, DH, KSPLIT, false>(p, stream) : launch_ring_r<M, DH, KSPLIT, true>(p, stream);
 }
 
 hipError_t launch_attn_ring(const AttnParams& p, int Dh, int dtype, int ksplit, hipStream_t stream) {

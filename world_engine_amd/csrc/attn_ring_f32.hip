@@ -74,8 +74,9 @@ __global__ void __launch_bounds__(256) attn_ring_f32_kernel(AttnParams p) {
       __syncthreads();  // the previous tile is no longer read
       for (int i = tid; i < TK * DH / 4; i += 256) {
         const int r = i / (DH / 4), c = i % (DH / 4);
-        *reinterpret_cast<f32x4_t*>(&ks[r][4 * c]) = *reinterpret_cast<const f32x4_t*>(kplane + (row0 + t0 + r) * DH + 4 * c);
-        *reinterpret_cast<f32x4_t*>(&vs[r][4 * c]) = *reinterpret_cast<const f32x4_t*>(vplane + (row0 + t0 + r) * DH + 4 * c);
+        const int tr = t0 + r < p.T ? t0 + r : p.T - 1;  // a short last tile repeats its last row; masked below
+        *reinterpret_cast<f32x4_t*>(&ks[r][4 * c]) = *reinterpret_cast<const f32x4_t*>(kplane + (row0 + tr) * DH + 4 * c);
+        *reinterpret_cast<f32x4_t*>(&vs[r][4 * c]) = *reinterpret_cast<const f32x4_t*>(vplane + (row0 + tr) * DH + 4 * c);
       }
       __syncthreads();
       float s[TK];
@@ -87,6 +88,7 @@ __global__ void __launch_bounds__(256) attn_ring_f32_kernel(AttnParams p) {
         for (int d = 0; d < PART; ++d) acc += q[d] * ks[kk][part * PART + d];
         acc += __shfl_xor(acc, 1);
         acc += __shfl_xor(acc, 2);
+        if (t0 + kk >= p.T) acc = -INFINITY;
         s[kk] = acc;
         mx = fmaxf(mx, acc);
       }

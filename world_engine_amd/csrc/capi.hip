@@ -131,7 +131,7 @@ int prepare_attn(const void* q, const int64_t* q_strides, const void* kv, const 
   if (rc != WE_OK) return rc;
   if (dtype != WE_DTYPE_BF16 && dtype != WE_DTYPE_F16 && dtype != WE_DTYPE_F32) return WE_ERR_UNSUPPORTED;
   if (Dh != 64 && Dh != 128) return WE_ERR_UNSUPPORTED;
-  if (T % 64 != 0 || L / T > WE_MAX_SLOTS) return WE_ERR_UNSUPPORTED;
+  if (L / T > WE_MAX_SLOTS) return WE_ERR_UNSUPPORTED;
   if ((uint64_t)(L + T) * (uint64_t)Dh * 2u >= (1ull << 32)) return WE_ERR_UNSUPPORTED;  // 32-bit tile offsets
   if (!(scale > 0.f) || n_splits < 0 || n_splits > 64) return WE_ERR_BAD_SHAPE;
   if (variant_of(q_tile) < 0) return WE_ERR_UNSUPPORTED;
