@@ -3,7 +3,7 @@
 
 A *step* is one frame-step of one attention layer: the fused RoPE + ring-slot K/V store followed
 by the attention over the ring (one we_rope_kv_store call + one we_attn_ring_fwd call through the
-C ABI).  The default workload is BASELINE config 1 (B=1, H=16, Dh=128, 256 tokens per frame,
+C ABI).  The default workload is benchmark configuration 1 (B=1, H=16, Dh=128, 256 tokens per frame,
 16-slot ring, bf16); ``--config 2|3|4`` select the other single-GPU configurations.  Inputs are
 synthetic N(0,1) tensors already resident in HBM, laid out like the merged QKV projection output.
 The timed region replays a HIP graph holding exactly K consecutive steps (the ring advances every

@@ -110,14 +110,14 @@ def _run_and_check(p, steps, frozen_subs=0, check_steps=None, outlier=False, lay
 
 
 def test_attention_cfg0_shapes_bf16(gpu_device):
-    """BASELINE config 0 geometry (B=1,H=8,Dh=64,T=64, 4 slots, 8 steps) in bf16 on the GPU."""
+    """Benchmark configuration 0 geometry (B=1,H=8,Dh=64,T=64, 4 slots, 8 steps) in bf16 on the GPU."""
     p = Pair(gpu_device, torch.bfloat16, B=1, H=8, Hkv=8, T=64, Dh=64, n_slots=4, cfg_id=0)
     worst = _run_and_check(p, 8)
     _say(f"cfg0 shapes: worst max-abs {worst[0]:.2e} mean-abs {worst[1]:.2e}")
 
 
 def test_attention_cfg0_fp32(gpu_device):
-    """BASELINE config 0 as stated (fp32, B=1, H=8, Dh=64, 64-token frames, 4 slots, 8 steps, the
+    """Benchmark configuration 0 as stated (fp32, B=1, H=8, Dh=64, 64-token frames, 4 slots, 8 steps, the
     ring wraps twice) through the fp32 kernel: fp32 arithmetic throughout, so the bar is 1e-5."""
     p = Pair(gpu_device, torch.float32, B=1, H=8, Hkv=8, T=64, Dh=64, n_slots=4, cfg_id=0)
     p.set_frozen(False)
@@ -146,7 +146,7 @@ def test_attention_fp32_other_shapes(gpu_device, Dh, hkv, T):
 
 
 def test_attention_cfg1_all_32_steps(gpu_device):
-    """BASELINE config 1: B=1,H=16,Dh=128,T=256, 16 slots, 32 steps (warm-up + steady wrap)."""
+    """Benchmark configuration 1: B=1,H=16,Dh=128,T=256, 16 slots, 32 steps (warm-up + steady wrap)."""
     p = Pair(gpu_device, torch.bfloat16, B=1, H=16, Hkv=16, T=256, Dh=128, n_slots=16, cfg_id=1)
     worst = _run_and_check(p, 32)
     _say(f"cfg1: worst max-abs {worst[0]:.2e} mean-abs {worst[1]:.2e}")
@@ -210,7 +210,7 @@ def test_attention_with_pinned_dilation(gpu_device, d):
 
 
 def test_attention_cfg2_outlier_channel_three_layers(gpu_device):
-    """BASELINE config 2 semantics (each layer its own ring, K with one x8 channel) on 3 layers."""
+    """Benchmark configuration 2 semantics (each layer its own ring, K with one x8 channel) on 3 layers."""
     p = Pair(gpu_device, torch.bfloat16, B=1, H=16, Hkv=16, T=256, Dh=128, n_slots=16, n_layers=3, cfg_id=2)
     p.set_frozen(False)
     for t in (0, 1, 2, 17):
@@ -223,7 +223,7 @@ def test_attention_cfg2_outlier_channel_three_layers(gpu_device):
 
 
 def test_attention_cfg4_frozen_substeps_schedule(gpu_device):
-    """BASELINE config 4: 32 slots, 4 frozen substeps re-attending the same ring + 1 persisting
+    """Benchmark configuration 4: 32 slots, 4 frozen substeps re-attending the same ring + 1 persisting
     call per frame.  State is compared after every call; outputs on the first frames and around
     the wrap."""
     p = Pair(gpu_device, torch.bfloat16, B=1, H=16, Hkv=16, T=256, Dh=128, n_slots=32, cfg_id=4)
@@ -231,7 +231,7 @@ def test_attention_cfg4_frozen_substeps_schedule(gpu_device):
 
 
 def test_attention_cfg3_full_size(gpu_device):
-    """BASELINE config 3 at full size (B=4,H=24,T=1024, 8 slots): oracle on three steps, plus
+    """Benchmark configuration 3 at full size (B=4,H=24,T=1024, 8 slots): oracle on three steps, plus
     size-independent properties on the steady state."""
     p = Pair(gpu_device, torch.bfloat16, B=4, H=24, Hkv=24, T=1024, Dh=128, n_slots=8, cfg_id=3)
     _run_and_check(p, 10, check_steps={0, 9})

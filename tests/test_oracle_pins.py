@@ -263,7 +263,7 @@ def _run_steps(dtype, B, H, Hkv, T, Dh, n_slots, steps, cfg_id=0, d=1):
 
 
 def test_cfg0_cpu_plumbing_fp32_against_flex_and_fp64():
-    """BASELINE config 0: B=1,H=8,Dh=64,T=64, 4 slots, fp32, 8 steps (ring wraps twice)."""
+    """Benchmark configuration 0: B=1,H=8,Dh=64,T=64, 4 slots, fp32, 8 steps (ring wraps twice)."""
     for s, q, k_all, v_all, mask in _run_steps(torch.float32, 1, 8, 8, 64, 64, 4, 8):
         assert int(mask.sum()) == min(s, 3) * 64 + 64
         ref_path = ro.attention_reference_path(q, k_all, v_all, mask)
