@@ -153,13 +153,41 @@ int we_attn_ring_fwd(const void* q, const int64_t q_strides[3],
                      int32_t dtype, void* stream);
 
 /*
+ * Optional work of the reference's attention module that sits right in front of and right behind
+ * the path and touches the same tiles (src/model/attn.py:105-109,117-119): done inside the two
+ * kernels instead of as five to seven element-wise launches per layer.  A zeroed struct (or a
+ * NULL pointer to one) switches everything off.
+ *   qk_norm_eps  > 0: q and k rows are RMS-normalised without weight before RoPE,
+ *                x * rsqrt(mean(x^2) + eps) in fp32, rounded to the element type (F.rms_norm;
+ *                torch uses the fp32 machine epsilon for low-precision inputs).  Needs Dh / 16 to
+ *                be a power of two <= 64.
+ *   v1, v_lamb   v = lerp(v, v1, *v_lamb) before the store (value residual); v1 [B, Hkv, T, Dh]
+ *                with element strides v1_strides = {batch, head, token}, v_lamb a device pointer
+ *                to one element.  Both NULL = off.
+ *   gate         out[b, h, t, :] *= gate[b, h, t] (sigmoid already applied), element strides
+ *                gate_strides = {batch, head, token}; the attention output is rounded to the
+ *                element type first, as the module's own multiply sees it.  NULL = off.
+ * Results equal the separate torch operations up to the last bit of the row reduction and of the
+ * lerp's fused multiply-add (1 ulp of the element type); the gate multiply is exact.
+ */
+typedef struct we_attn_extras {
+  float qk_norm_eps;
+  const void* v1;
+  int64_t v1_strides[3];
+  const void* v_lamb;
+  const void* gate;
+  int64_t gate_strides[3];
+} we_attn_extras;
+
+/*
  * RoPE + K/V store + attention of one frame in a single call: we_rope_kv_store followed by
  * we_attn_ring_fwd on the rotated q, i.e. the whole per-layer sequence of the reference from
  * `q, k = rope(q), rope(k)` to the flex_attention call (src/model/attn.py:110-116 with
  * src/model/kv_cache.py:126-151).  Arguments, requirements and results (cache rows, `written`,
  * q_out, out) are those of the two calls, bit for bit; q, q_out and the tables are mandatory.
  * Both calls are validated before anything is launched, and a host language pays for one
- * foreign call per layer and frame instead of two.
+ * foreign call per layer and frame instead of two.  `extras` (may be NULL) adds the module's
+ * element-wise neighbours of the path, see we_attn_extras; q_out then holds RoPE(rms_norm(q)).
  */
 int we_rope_kv_attn_fwd(const void* q, const void* k, const void* v,
                         const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
@@ -172,7 +200,7 @@ int we_rope_kv_attn_fwd(const void* q, const void* k, const void* v,
                         void* workspace, size_t workspace_bytes,
                         int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L,
                         int32_t dilation, int32_t is_frozen, float scale, int32_t n_splits, int32_t q_tile,
-                        int32_t dtype, void* stream);
+                        int32_t dtype, const we_attn_extras* extras, void* stream);
 
 #ifdef __cplusplus
 }

@@ -173,7 +173,7 @@ def test_one_call_entry_point_validates_both_halves():
     args = lambda **kw: [kw.get("q", fake), fake, fake, s3, s3, s3, kw.get("q_out", fake), kw.get("cos", fake), fake, 10,
                          fake, fake, fake, 64, 8, 8, fake, fake, kw.get("out", fake), s3, None, 0,
                          1, 1, 1, 64, kw.get("Dh", 64), kw.get("L", 64), 1, 0, 0.1, kw.get("n_splits", 1), 0,
-                         kw.get("dtype", 0), None]
+                         kw.get("dtype", 0), kw.get("extras"), None]
     assert lib.we_rope_kv_attn_fwd(*args(q=None)) == -1
     assert lib.we_rope_kv_attn_fwd(*args(q_out=None)) == -1
     assert lib.we_rope_kv_attn_fwd(*args(cos=None)) == -1
@@ -183,6 +183,13 @@ def test_one_call_entry_point_validates_both_halves():
     assert lib.we_rope_kv_attn_fwd(*args(dtype=2, n_splits=2)) == -3 # fp32 runs the one-pass kernel only
     assert lib.we_rope_kv_attn_fwd(*args(dtype=3)) == -3
     assert lib.we_rope_kv_attn_fwd(*args(n_splits=2)) == -5          # splits without workspace
+    # extras: lerp needs both the residual and its weight; negative epsilon; norm needs Dh/16 a power of two
+    ex = _capi.AttnExtras()
+    ex.v1 = 4096
+    assert lib.we_rope_kv_attn_fwd(*args(extras=ctypes.byref(ex))) == -1
+    ex = _capi.AttnExtras()
+    ex.qk_norm_eps = -1.0
+    assert lib.we_rope_kv_attn_fwd(*args(extras=ctypes.byref(ex))) == -2
 
 
 def test_attention_kernels_keep_their_state_in_registers():

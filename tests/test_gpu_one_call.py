@@ -112,3 +112,89 @@ def test_module_forward_compiles_as_one_graph(gpu_device):
         assert torch.equal(y_e, y_c), f"t={t}"
         assert_bits_equal(caches[0].layers[0].kv, caches[1].layers[0].kv, f"cache t={t}")
         assert torch.equal(caches[0].layers[0].written, caches[1].layers[0].written)
+
+
+def _ulp_close(a, b, what, ulps=1):
+    """Element-type tensors equal up to `ulps` units in the last place of the largest value of
+    their row (a last-bit difference in a normalised input moves a rotated pair, a difference of
+    products, by that much whatever the size of the result).  Returns the fraction that differs."""
+    a32, b32 = a.float().cpu(), b.float().cpu()
+    eps = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}[a.dtype]
+    tol = 2 * ulps * eps * b32.abs().amax(dim=-1, keepdim=True).clamp_min(2.0 ** -100)
+    bad = (a32 - b32).abs() > tol
+    assert not bad.any(), f"{what}: {int(bad.sum())} elements off by more than {ulps} ulp of their row's largest"
+    return float((a32 != b32).float().mean())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_fused_neighbours_match_torch_ops(gpu_device, dtype):
+    """qk RMS norm, value-residual lerp and head gate inside the kernels against the same torch
+    operations in front of / behind the plain call: cache rows and RoPE(q) within 1 ulp (and
+    mostly identical), `written` identical, gated output within the attention bar."""
+    dev = gpu_device
+    B, H, Hkv, T, Dh, n = 2, 4, 2, 128, 128, 3
+    p_f = Pair(dev, dtype, B=B, H=H, Hkv=Hkv, T=T, Dh=Dh, n_slots=n, cfg_id=61)     # fused
+    p_u = Pair(dev, dtype, B=B, H=H, Hkv=Hkv, T=T, Dh=Dh, n_slots=n, cfg_id=61)     # torch ops + plain call
+    eps = torch.finfo(torch.float32).eps
+    g = torch.Generator("cpu").manual_seed(7)
+    lamb = torch.tensor(0.37, dtype=dtype, device=dev)
+    for t in range(7):
+        frozen = t % 3 == 1
+        q, k, v, pos = p_f.inputs(t)
+        v1 = torch.randn(v.shape, generator=g).to(dtype)
+        gate = torch.sigmoid(torch.randn(B, T, H, generator=g)).to(dtype).to(dev).permute(0, 2, 1)   # strided [B,H,T]
+        qd, kd, vd = merged_views(q.to(dev), k.to(dev), v.to(dev))
+        v1d = v1.to(dev)
+        posd = to_dev(pos, dev)
+        lf, lu = p_f.hip.layers[0], p_u.hip.layers[0]
+        out_f, qrot_f = ops.rope_kv_attn(qd, kd, vd, posd, p_f.rope.cos, p_f.rope.sin, p_f.rope.height, p_f.rope.width,
+                                         lf.kv, lf.written, lf.L, 1, frozen, qk_norm_eps=eps, v1=v1d, v_lamb=lamb,
+                                         gate=gate)
+        qn = torch.nn.functional.rms_norm(qd, (Dh,))
+        kn = torch.nn.functional.rms_norm(kd, (Dh,))
+        vl = torch.lerp(vd, v1d, lamb)
+        out_u, qrot_u = ops.rope_kv_attn(qn, kn, vl, posd, p_u.rope.cos, p_u.rope.sin, p_u.rope.height, p_u.rope.width,
+                                         lu.kv, lu.written, lu.L, 1, frozen)
+        out_u = out_u * gate.unsqueeze(-1)
+        frac = _ulp_close(qrot_f, qrot_u, f"RoPE(norm(q)) t={t}")
+        frac_kv = _ulp_close(lf.kv, lu.kv, f"cache t={t}")
+        assert frac < 0.02 and frac_kv < 0.02, (frac, frac_kv)
+        assert torch.equal(lf.written, lu.written)
+        assert_attn_close(out_f, out_u.float().cpu(), f"gated output t={t}")
+
+
+def test_module_with_fused_neighbours(gpu_device):
+    """RingAttn(fuse_elementwise=True) against the same module with the torch operations."""
+    import types
+    import world_engine_amd as wea
+    torch.manual_seed(1)
+    cfg = types.SimpleNamespace(d_model=512, n_heads=4, n_kv_heads=4, value_residual=True, gated_attn=True,
+                                tokens_per_frame=64, local_window=3, global_window=3, global_attn_period=1,
+                                global_pinned_dilation=1, n_layers=2)
+    cos, sin = ro.rope_table_1d(16 * 64, 128)
+    rope = wea.RoPE(cos, sin, 8, 8).to(gpu_device)
+    plain = [wea.RingAttn(cfg, i, rope, merged_qkv=True).to(gpu_device, torch.bfloat16) for i in range(2)]
+    fused = [wea.RingAttn(cfg, i, rope, merged_qkv=True, fuse_elementwise=True).to(gpu_device, torch.bfloat16)
+             for i in range(2)]
+    for a, b in zip(plain, fused):
+        with torch.no_grad():
+            a.gate_proj.weight.normal_(0, 0.5)
+            a.v_lamb.fill_(0.3)
+        b.load_state_dict(a.state_dict())
+    caches = [wea.StaticKVCache(cfg, 1, torch.bfloat16).to(gpu_device) for _ in range(2)]
+    for c in caches:
+        c.set_frozen(False)
+    for t in range(5):
+        x = torch.randn(1, 64, 512, device=gpu_device, dtype=torch.bfloat16)
+        pos = to_dev(ro.synth_pos_ids(t, 1, 64, 8), gpu_device)
+        with torch.no_grad():
+            ya, v1a = plain[0](x, pos, None, caches[0])
+            ya2, _ = plain[1](ya, pos, v1a, caches[0])
+            yb, v1b = fused[0](x, pos, None, caches[1])
+            yb2, _ = fused[1](yb, pos, v1b, caches[1])
+        d1 = (ya.float() - yb.float()).abs().max().item()
+        d2 = (ya2.float() - yb2.float()).abs().max().item()
+        scale = ya2.float().abs().max().item()
+        assert d1 <= 2e-2 * max(1.0, ya.float().abs().max().item()) and d2 <= 3e-2 * max(1.0, scale), (t, d1, d2)
+        for li in range(2):
+            _ulp_close(caches[1].layers[li].kv, caches[0].layers[li].kv, f"layer {li} cache t={t}", ulps=2 if li else 1)

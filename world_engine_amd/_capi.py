@@ -17,6 +17,12 @@ WE_MAX_SLOTS = 256
 
 _I64x3 = POINTER(c_int64)
 
+class AttnExtras(ctypes.Structure):
+    """``we_attn_extras`` of include/we_attn.h."""
+    _fields_ = [("qk_norm_eps", ctypes.c_float), ("v1", c_void_p), ("v1_strides", ctypes.c_int64 * 3),
+                ("v_lamb", c_void_p), ("gate", c_void_p), ("gate_strides", ctypes.c_int64 * 3)]
+
+
 # name -> (restype, argtypes); must list every symbol include/we_attn.h declares
 SIGNATURES = {
     "we_version": (c_int32, []),
@@ -61,7 +67,8 @@ SIGNATURES = {
         c_void_p, _I64x3,                          # out, out_strides
         c_void_p, c_size_t,                        # workspace, bytes
         c_int32, c_int32, c_int32, c_int32, c_int32, c_int64,   # B H Hkv T Dh L
-        c_int32, c_int32, c_float, c_int32, c_int32, c_int32, c_void_p,  # dilation frozen scale n_splits q_tile dtype stream
+        c_int32, c_int32, c_float, c_int32, c_int32, c_int32,  # dilation frozen scale n_splits q_tile dtype
+        c_void_p, c_void_p,                        # extras (we_attn_extras* or NULL), stream
     ]),
 }
 

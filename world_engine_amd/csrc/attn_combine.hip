@@ -56,8 +56,14 @@ __global__ void __launch_bounds__(256) attn_combine_kernel(AttnParams p) {
   const unsigned bh = (unsigned)(p.units_whole * p.group) + blockIdx.y;  // first split pair + y
   const int b = (int)(bh / (unsigned)p.H), h = (int)(bh % (unsigned)p.H);
   uint16_t* dst = reinterpret_cast<uint16_t*>(p.out) + b * p.os_b + h * p.os_h + (int64_t)t * p.os_t + dg * 8;
-  *reinterpret_cast<frag_t*>(dst) = M::pack8(acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv, acc[4] * inv,
-                                             acc[5] * inv, acc[6] * inv, acc[7] * inv);
+  frag_t y = M::pack8(acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv, acc[4] * inv, acc[5] * inv,
+                      acc[6] * inv, acc[7] * inv);
+  if (p.gate != nullptr) {  // y * gate on element-type values, as the module's own multiply
+    const float g = (float)reinterpret_cast<const typename M::elem_t*>(p.gate)[b * p.gs_b + h * p.gs_h + (int64_t)t * p.gs_t];
+    y = M::pack8((float)y[0] * g, (float)y[1] * g, (float)y[2] * g, (float)y[3] * g, (float)y[4] * g,
+                 (float)y[5] * g, (float)y[6] * g, (float)y[7] * g);
+  }
+  *reinterpret_cast<frag_t*>(dst) = y;
 }
 
 hipError_t launch_attn_combine(const AttnParams& p, int Dh, int dtype, hipStream_t stream) {

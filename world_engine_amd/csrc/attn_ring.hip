@@ -663,6 +663,9 @@ attn_ring_kernel(AttnParams p) {
   const bool valid = qrow < p.T;
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   const int64_t row = ((int64_t)b * p.H + h) * p.T + qrow;
+  float gate_v = 1.f;
+  if (p.gate != nullptr && nsp == 1 && qrow < p.T)
+    gate_v = (float)reinterpret_cast<const typename M::elem_t*>(p.gate)[b * p.gs_b + h * p.gs_h + (int64_t)qrow * p.gs_t];
   if (nsp > 1 && valid && hh == 0) {
     float2 ml = make_float2(m_ref, l_tot);
     *reinterpret_cast<float2*>(p.ws_ml + ((int64_t)split * rows + (row - p.ws_row0)) * 2) = ml;
@@ -686,7 +689,12 @@ attn_ring_kernel(AttnParams p) {
         if (nsp == 1) {
           uint16_t* dst = reinterpret_cast<uint16_t*>(p.out) + b * p.os_b + h * p.os_h +
                           (int64_t)qrow * p.os_t + d0;
-          *reinterpret_cast<frag_t*>(dst) = M::pack8(f[0], f[1], f[2], f[3], f[4], f[5], f[6], f[7]);
+          frag_t y = M::pack8(f[0], f[1], f[2], f[3], f[4], f[5], f[6], f[7]);
+          if (p.gate != nullptr) {  // y * gate on element-type values, as the module's own multiply
+            y = M::pack8((float)y[0] * gate_v, (float)y[1] * gate_v, (float)y[2] * gate_v, (float)y[3] * gate_v,
+                         (float)y[4] * gate_v, (float)y[5] * gate_v, (float)y[6] * gate_v, (float)y[7] * gate_v);
+          }
+          *reinterpret_cast<frag_t*>(dst) = y;
         } else {
           uint16_t* dst = p.ws_o + ((int64_t)split * rows + (row - p.ws_row0)) * DH + d0;
           *reinterpret_cast<frag_t*>(dst) = M::pack8(f[0], f[1], f[2], f[3], f[4], f[5], f[6], f[7]);

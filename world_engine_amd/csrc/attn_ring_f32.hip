@@ -108,11 +108,13 @@ __global__ void __launch_bounds__(256) attn_ring_f32_kernel(AttnParams p) {
   }
 
   if (qrow < p.T) {
-    const float inv = 1.f / l_run;
+    float inv = 1.f / l_run;
+    // fp32: o * inv is the attention output; the gate multiplies that rounded value
+    const float g = p.gate != nullptr ? reinterpret_cast<const float*>(p.gate)[b * p.gs_b + h * p.gs_h + (int64_t)qrow * p.gs_t] : 1.f;
     float* dst = reinterpret_cast<float*>(p.out) + b * p.os_b + h * p.os_h + (int64_t)qrow * p.os_t + part * PART;
 #pragma unroll
     for (int d = 0; d < PART; d += 4)
-      *reinterpret_cast<f32x4_t*>(dst + d) = f32x4_t{o[d] * inv, o[d + 1] * inv, o[d + 2] * inv, o[d + 3] * inv};
+      *reinterpret_cast<f32x4_t*>(dst + d) = f32x4_t{(o[d] * inv) * g, (o[d + 1] * inv) * g, (o[d + 2] * inv) * g, (o[d + 3] * inv) * g};
   }
 }
 

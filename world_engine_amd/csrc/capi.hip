@@ -118,6 +118,7 @@ int prepare_store(const void* q, const void* k, const void* v, const int64_t* q_
   p.L = L;
   p.B = B; p.H = H; p.Hkv = Hkv; p.T = T; p.Dh = Dh;
   p.dilation = dilation; p.num_buckets = (int)((L / T) / dilation); p.frozen = is_frozen ? 1 : 0;
+  p.norm_eps = 0.f; p.v1 = nullptr; p.v_lamb = nullptr; p.v1s_b = p.v1s_h = p.v1s_t = 0;
   return WE_OK;
 }
 
@@ -167,6 +168,7 @@ int prepare_attn(const void* q, const int64_t* q_strides, const void* kv, const 
   p.members = p.group * p.q_tiles;
   p.unit_splits = pl.units_whole + (B * Hkv - pl.units_whole) * pl.n_splits;
   p.scale_log2 = scale * 1.4426950408889634f;
+  p.gate = nullptr; p.gs_b = p.gs_h = p.gs_t = 0;
 
   if ((p.unit_splits + 7) / 8 > 65535 || p.group > 65535 || (int64_t)B * H - (int64_t)pl.units_whole * p.group > 65535)
     return WE_ERR_UNSUPPORTED;  // grid y / z limits of the two launches
@@ -281,7 +283,7 @@ int we_rope_kv_attn_fwd(const void* q, const void* k, const void* v, const int64
                         const int64_t out_strides[3], void* workspace, size_t workspace_bytes, int32_t B,
                         int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L, int32_t dilation,
                         int32_t is_frozen, float scale, int32_t n_splits, int32_t q_tile, int32_t dtype,
-                        void* stream) {
+                        const we_attn_extras* extras, void* stream) {
   if (!q || !q_out || !cos_table) return WE_ERR_NULL_POINTER;
   we::StoreParams sp;
   int rc = prepare_store(q, k, v, q_strides, k_strides, v_strides, q_out, cos_table, sin_table, table_rows, t_pos,
@@ -295,6 +297,18 @@ int we_rope_kv_attn_fwd(const void* q, const void* k, const void* v, const int64
   rc = prepare_attn(q_out, qo_strides, kv, written, t_pos, out, out_strides, workspace, workspace_bytes, B, H, Hkv,
                     T, Dh, L, dilation, scale, n_splits, q_tile, dtype, p, pl);
   if (rc != WE_OK) return rc;
+  if (extras) {
+    const we_attn_extras& x = *extras;
+    if (x.qk_norm_eps < 0.f || x.qk_norm_eps != x.qk_norm_eps) return WE_ERR_BAD_SHAPE;
+    if (x.qk_norm_eps > 0.f && (sp.cpr_shift < 0 || (Dh >> 4) > 64)) return WE_ERR_UNSUPPORTED;
+    if ((x.v1 == nullptr) != (x.v_lamb == nullptr)) return WE_ERR_NULL_POINTER;
+    if (x.v1 && (!aligned16(x.v1) || !strides_ok(x.v1_strides, dtype))) return WE_ERR_ALIGNMENT;
+    sp.norm_eps = x.qk_norm_eps;
+    sp.v1 = x.v1; sp.v_lamb = x.v_lamb;
+    sp.v1s_b = x.v1_strides[0]; sp.v1s_h = x.v1_strides[1]; sp.v1s_t = x.v1_strides[2];
+    p.gate = x.gate;
+    p.gs_b = x.gate_strides[0]; p.gs_h = x.gate_strides[1]; p.gs_t = x.gate_strides[2];
+  }
   hipStream_t st = static_cast<hipStream_t>(stream);
   // Everything is validated before the first launch; the kernels follow each other on the stream.
   if (we::launch_rope_kv_store(sp, dtype, st) != hipSuccess) return WE_ERR_LAUNCH;

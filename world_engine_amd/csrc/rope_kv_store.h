@@ -64,6 +64,36 @@ __device__ __forceinline__ void store8(void* p, const Chunk8<Tag>& c) {
   for (int i = 0; i < nvec; ++i) dst[i] = src[i];
 }
 
+// Weightless RMS norm of a row held 16 elements per lane by `cpr` consecutive lanes (a power of
+// two, at most 64): x * rsqrt(mean(x^2) + eps) in fp32, rounded to the element type, as
+// F.rms_norm on a low-precision tensor does (src/model/nn.py:55-56).
+template <typename Tag>
+__device__ __forceinline__ void rms_norm_chunk(Chunk16<Tag>& c, int cpr, int Dh, float eps) {
+  float x[16];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    x[i] = Tag::to_f32(c.e[i]);
+    ss += x[i] * x[i];
+  }
+  for (int m = 1; m < cpr; m <<= 1) ss += __shfl_xor(ss, m);
+  const float r = rsqrtf(ss / (float)Dh + eps);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) c.e[i] = Tag::from_f32(x[i] * r);
+}
+
+// torch.lerp(v, v1, w) on 16 elements: fp32 arithmetic, the formula switches at w = 0.5
+// (ATen/native/Lerp.h), result rounded to the element type.
+template <typename Tag>
+__device__ __forceinline__ void lerp_chunk(Chunk16<Tag>& v, const Chunk16<Tag>& v1, float w) {
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const float a = Tag::to_f32(v.e[i]), b = Tag::to_f32(v1.e[i]);
+    const float d = b - a;
+    v.e[i] = Tag::from_f32(w < 0.5f ? a + w * d : b - d * (1.f - w));
+  }
+}
+
 // Row of the cos / sin tables for token t of batch element b (src/model/attn.py:33-36): the
 // three position ids select one row of the flattened [frames, height, width] table.
 __device__ __forceinline__ int64_t rope_table_row(const StoreParams& p, int b, int t) {
@@ -151,6 +181,12 @@ __device__ __forceinline__ void store_kv_item(const StoreParams& p, int which, i
                                : (const st_t*)p.v + b * p.vs_b + h * p.vs_h + t * p.vs_t;
   Chunk16<Tag> in;
   load16<Tag>(in, src + chunk * 16);
+  if (which == 1 && p.norm_eps > 0.f) rms_norm_chunk<Tag>(in, p.Dh >> 4, p.Dh, p.norm_eps);
+  if (which == 2 && p.v1 != nullptr) {
+    Chunk16<Tag> res;
+    load16<Tag>(res, (const st_t*)p.v1 + b * p.v1s_b + h * p.v1s_h + t * p.v1s_t + chunk * 16);
+    lerp_chunk<Tag>(in, res, Tag::to_f32(*reinterpret_cast<const st_t*>(p.v_lamb)));
+  }
   const bool rotate = which == 1 && p.cos_t != nullptr;
   Chunk8<Tag> lo, hi;
   if (rotate) {

@@ -42,6 +42,7 @@ __global__ void __launch_bounds__(256) rope_kv_store_kernel(StoreParams p) {
   const int h = head_all;
   Chunk16<Tag> in;
   load16<Tag>(in, (const st_t*)p.q + b * p.qs_b + h * p.qs_h + t * p.qs_t + chunk * 16);
+  if (p.norm_eps > 0.f) rms_norm_chunk<Tag>(in, cpr, p.Dh, p.norm_eps);
   st_t* dst = (st_t*)p.q_out + (((int64_t)b * p.H + h) * p.T + t) * p.Dh;
   if (p.cos_t != nullptr) {
     const int64_t pos = rope_table_row(p, b, t);

@@ -28,6 +28,11 @@ struct StoreParams {
   int B, H, Hkv, T, Dh;
   int dilation, num_buckets, frozen;
   int cpr_shift;  // log2(Dh / 16) when Dh / 16 is a power of two, else -1
+  // optional work of the attention module in front of RoPE (src/model/attn.py:105-109)
+  float norm_eps;             // > 0: q and k rows are RMS-normalised (no weight) first
+  const void* v1;             // value residual [B, Hkv, T, Dh] or null: v = lerp(v, v1, *v_lamb)
+  const void* v_lamb;         // device pointer to the lerp weight, element type
+  int64_t v1s_b, v1s_h, v1s_t;
 };
 
 struct AttnParams {
@@ -51,6 +56,9 @@ struct AttnParams {
   int members;      // workgroups that share one K/V stream: group * q_tiles
   int unit_splits;  // units_whole + (B * Hkv - units_whole) * n_splits
   float scale_log2; // softmax scale * log2(e)
+  // optional per (batch, head, token) output gate, element type (src/model/attn.py:117-119)
+  const void* gate;
+  int64_t gs_b, gs_h, gs_t;
 };
 
 hipError_t launch_rope_kv_store(const StoreParams& p, int dtype, hipStream_t stream);

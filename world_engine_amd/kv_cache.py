@@ -114,7 +114,9 @@ class LayerKVCache(nn.Module):
         return q_rot, self.kv[0], self.kv[1], self._mask(pos_ids)
 
     def rope_upsert_attend(self, q: Tensor, k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor], rope,
-                           is_frozen: bool, scale: Optional[float] = None) -> Tensor:
+                           is_frozen: bool, scale: Optional[float] = None, qk_norm_eps: float = 0.0,
+                           v1: Optional[Tensor] = None, v_lamb: Optional[Tensor] = None,
+                           gate: Optional[Tensor] = None) -> Tensor:
         """``rope_upsert`` followed by the attention over the ring, as one library call
         (``src/model/attn.py:110-116`` of the reference from RoPE to ``flex_attention``).  Under
         ``torch.compile`` the registered opaque op is used instead of the eager wrapper."""
@@ -122,10 +124,12 @@ class LayerKVCache(nn.Module):
             s = float(scale) if scale is not None else float(q.shape[-1]) ** -0.5
             return torch.ops.world_engine_amd.rope_kv_attn(
                 q, k, v, pos_ids["t_pos"], pos_ids["y_pos"], pos_ids["x_pos"], rope.cos, rope.sin, rope.height,
-                rope.width, self.kv, self.written, self.L, self.pinned_dilation, bool(is_frozen), s)
+                rope.width, self.kv, self.written, self.L, self.pinned_dilation, bool(is_frozen), s,
+                float(qk_norm_eps), v1, v_lamb, gate)
         self._check(k, pos_ids)
         return ops.rope_kv_attn(q, k, v, pos_ids, rope.cos, rope.sin, rope.height, rope.width, self.kv,
-                                self.written, self.L, self.pinned_dilation, is_frozen, scale)[0]
+                                self.written, self.L, self.pinned_dilation, is_frozen, scale,
+                                qk_norm_eps=qk_norm_eps, v1=v1, v_lamb=v_lamb, gate=gate)[0]
 
 
 class StaticKVCache(nn.Module):
@@ -162,5 +166,5 @@ class StaticKVCache(nn.Module):
         return self.layers[layer].rope_upsert(q, k, v, pos_ids, rope, self._is_frozen)
 
     def rope_upsert_attend(self, q: Tensor, k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor], rope, layer: int,
-                           scale: Optional[float] = None) -> Tensor:
-        return self.layers[layer].rope_upsert_attend(q, k, v, pos_ids, rope, self._is_frozen, scale)
+                           scale: Optional[float] = None, **extras) -> Tensor:
+        return self.layers[layer].rope_upsert_attend(q, k, v, pos_ids, rope, self._is_frozen, scale, **extras)

@@ -6,6 +6,7 @@ on a ROCm device; anything else raises.
 """
 from __future__ import annotations
 
+import ctypes
 import math
 from typing import Mapping, Optional, Tuple
 
@@ -203,11 +204,19 @@ def rope_kv_attn(q: Tensor, k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor],
                  sin_table: Tensor, grid_h: int, grid_w: int, kv: Tensor, written: Tensor, L: int,
                  dilation: int, is_frozen: bool, scale: Optional[float] = None, n_splits: int = 0,
                  q_tile: int = 0, out: Optional[Tensor] = None, workspace: Optional[Tensor] = None,
-                 token_major_out: bool = True):
+                 token_major_out: bool = True, qk_norm_eps: float = 0.0, v1: Optional[Tensor] = None,
+                 v_lamb: Optional[Tensor] = None, gate: Optional[Tensor] = None):
     """``rope_kv_store`` followed by ``attn_ring`` in one library call (``we_rope_kv_attn_fwd``):
     the per-layer sequence of the reference from ``q, k = rope(q), rope(k)`` to the
     ``flex_attention`` call (``src/model/attn.py:110-116``), validated as a whole before the first
-    launch.  Returns ``(out, q_rot)``; results are those of the two separate calls, bit for bit."""
+    launch.  Returns ``(out, q_rot)``; results are those of the two separate calls, bit for bit.
+
+    Optional neighbours of the path done inside the kernels (``src/model/attn.py:105-109,117-119``):
+    ``qk_norm_eps > 0`` RMS-normalises q and k rows first (``F.rms_norm`` without weight; torch's
+    epsilon for low-precision inputs is ``torch.finfo(torch.float32).eps``); ``v1`` ``[B,Hkv,T,Dh]``
+    with the one-element ``v_lamb`` stores ``lerp(v, v1, v_lamb)``; ``gate`` ``[B,H,T]`` (any
+    strides, sigmoid applied) multiplies the output rows.  These match the separate torch operations
+    to 1 ulp of the element type (row reduction order, fused multiply-add in the lerp)."""
     dev = _need_device(q, k, v, kv, written, cos_table, sin_table, pos_ids["t_pos"])
     if k.dim() != 4 or k.shape != v.shape:
         raise RuntimeError("k and v must both be [B, Hkv, T, Dh]")
@@ -240,6 +249,23 @@ def rope_kv_attn(q: Tensor, k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor],
             out = torch.empty((B, H, T, Dh), dtype=q.dtype, device=dev)
     elif tuple(out.shape) != (B, H, T, Dh) or out.dtype != q.dtype or out.device != dev:
         raise RuntimeError("out must be [B, H, T, Dh] of q's element type on q's device")
+    extras = None
+    if qk_norm_eps or v1 is not None or gate is not None:
+        ex = _capi.AttnExtras()
+        ex.qk_norm_eps = float(qk_norm_eps)
+        if v1 is not None:
+            if v_lamb is None or v_lamb.numel() != 1 or v_lamb.dtype != v.dtype or v1.shape != v.shape or v1.dtype != v.dtype:
+                raise RuntimeError("v1 must match v and v_lamb must be one element of the same type")
+            _need_device(v1, v_lamb)
+            ex.v1, ex.v_lamb = v1.data_ptr(), v_lamb.data_ptr()
+            ex.v1_strides = _bhtd_strides(v1, "v1")
+        if gate is not None:
+            if tuple(gate.shape) != (B, H, T) or gate.dtype != q.dtype:
+                raise RuntimeError("gate must be [B, H, T] of q's element type")
+            _need_device(gate)
+            ex.gate = gate.data_ptr()
+            ex.gate_strides = _capi.i64x3(*gate.stride())
+        extras = ctypes.byref(ex)
     code = lib.we_rope_kv_attn_fwd(
         q.data_ptr(), k.data_ptr(), v.data_ptr(), _bhtd_strides(q, "q"), _bhtd_strides(k, "k"), _bhtd_strides(v, "v"),
         q_rot.data_ptr(), cos_table.data_ptr(), sin_table.data_ptr(), cos_table.shape[0],
@@ -248,7 +274,7 @@ def rope_kv_attn(q: Tensor, k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor],
         workspace.data_ptr() if ws_bytes else None,
         workspace.numel() * workspace.element_size() if ws_bytes else 0,
         B, H, Hkv, T, Dh, L, dilation, int(bool(is_frozen)), scale, n_splits, q_tile, _dtype_code(kv),
-        _stream_ptr(dev))
+        extras, _stream_ptr(dev))
     _capi.check(code, "we_rope_kv_attn_fwd")
     return out, q_rot
 
@@ -287,14 +313,16 @@ def _attn_ring_fake(q, kv, written, t_pos, L, dilation, scale):
 @torch.library.custom_op("world_engine_amd::rope_kv_attn", mutates_args=("kv", "written"))
 def rope_kv_attn_op(q: Tensor, k: Tensor, v: Tensor, t_pos: Tensor, y_pos: Tensor, x_pos: Tensor,
                     cos_table: Tensor, sin_table: Tensor, grid_h: int, grid_w: int,
-                    kv: Tensor, written: Tensor, L: int, dilation: int, is_frozen: bool, scale: float) -> Tensor:
+                    kv: Tensor, written: Tensor, L: int, dilation: int, is_frozen: bool, scale: float,
+                    qk_norm_eps: float = 0.0, v1: Optional[Tensor] = None, v_lamb: Optional[Tensor] = None,
+                    gate: Optional[Tensor] = None) -> Tensor:
     pos = {"t_pos": t_pos, "y_pos": y_pos, "x_pos": x_pos}
     return rope_kv_attn(q, k, v, pos, cos_table, sin_table, grid_h, grid_w, kv, written, L, dilation,
-                        is_frozen, scale)[0]
+                        is_frozen, scale, qk_norm_eps=qk_norm_eps, v1=v1, v_lamb=v_lamb, gate=gate)[0]
 
 
 @rope_kv_attn_op.register_fake
 def _rope_kv_attn_fake(q, k, v, t_pos, y_pos, x_pos, cos_table, sin_table, grid_h, grid_w, kv, written, L,
-                       dilation, is_frozen, scale):
+                       dilation, is_frozen, scale, qk_norm_eps=0.0, v1=None, v_lamb=None, gate=None):
     B, H, T, Dh = q.shape
     return q.new_empty((B, T, H, Dh)).transpose(1, 2)
