@@ -30,7 +30,16 @@
 // run on the matrix cores while the VALU handles block i); LDS fragment reads are stated up to 15
 // reads ahead of their MFMAs, also across steps and barriers, and the order is pinned with
 // sched_barrier.  When the workgroup count leaves a partial last round of CUs, only that round's
-// (batch, kv head) units are context-split (see the planner in capi.hip).
+// (batch, kv head) units are context-split (see the planner in capi.hip); split workgroups leave
+// normalised partial outputs that attn_combine.hip merges.
+//
+// The grid is 3-D (8 * query tiles, query heads per kv head, rounds of 8 units): no division by
+// run-time values is needed to find a workgroup's unit, and blockIdx.x % 8 is the XCD it runs on,
+// so the workgroups that share one K/V stream share an L2.  Start-up code is kept short on purpose:
+// a 256-token frame runs 8 tiles per workgroup and start-up is a third of the kernel.
+//
+// Frame lengths that are not a multiple of 64 use the RAGGED instantiation: the short last tile
+// of a slot is loaded with its missing rows clamped and its missing keys masked to -inf.
 //
 // Roofline: 4*T*N_vis*Dh flops and 4*N_vis*Dh bytes of K/V per (batch, kv head).
 #include "attn_mma.h"

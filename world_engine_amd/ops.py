@@ -71,6 +71,21 @@ def _pos_triplet(pos_ids: Mapping[str, Tensor], B: int, T: int, need_yx: bool):
     return t_pos, y_pos, x_pos, t_pos.stride(0)
 
 
+def _check_cache(kv: Tensor, written: Tensor, B: int, Hkv: int, T: int, Dh: int, L: int) -> None:
+    if kv.dim() != 5 or tuple(kv.shape) != (2, B, Hkv, L + T, Dh) or not kv.is_contiguous():
+        raise RuntimeError("kv must be a contiguous [2, B, Hkv, L+T, Dh] buffer; "
+                           "KV cache expects exactly one frame per upsert")
+    if written.dtype != torch.bool or written.numel() != L + T or not written.is_contiguous():
+        raise RuntimeError("written must be a contiguous bool [L+T] tensor")
+
+
+def _check_tables(cos_table: Tensor, sin_table: Tensor, Dh: int) -> None:
+    if (cos_table.dtype != torch.float32 or sin_table.dtype != torch.float32
+            or cos_table.shape != sin_table.shape or cos_table.dim() != 2 or cos_table.shape[1] != Dh // 2
+            or not cos_table.is_contiguous() or not sin_table.is_contiguous()):
+        raise RuntimeError("cos/sin tables must be contiguous fp32 [rows, Dh/2]")
+
+
 def rope_kv_store(q: Optional[Tensor], k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor],
                   cos_table: Optional[Tensor], sin_table: Optional[Tensor],
                   grid_h: int, grid_w: int, kv: Tensor, written: Tensor, L: int, dilation: int,
@@ -88,11 +103,7 @@ def rope_kv_store(q: Optional[Tensor], k: Tensor, v: Tensor, pos_ids: Mapping[st
     B, Hkv, T, Dh = k.shape
     if k.dtype != kv.dtype or v.dtype != kv.dtype or (q is not None and q.dtype != kv.dtype):
         raise RuntimeError("q/k/v must have the cache's element type")
-    if kv.dim() != 5 or tuple(kv.shape) != (2, B, Hkv, L + T, Dh) or not kv.is_contiguous():
-        raise RuntimeError("kv must be a contiguous [2, B, Hkv, L+T, Dh] buffer; "
-                           "KV cache expects exactly one frame per upsert")
-    if written.dtype != torch.bool or written.numel() != L + T or not written.is_contiguous():
-        raise RuntimeError("written must be a contiguous bool [L+T] tensor")
+    _check_cache(kv, written, B, Hkv, T, Dh, L)
     H = Hkv
     q_out = None
     if q is not None:
@@ -102,11 +113,7 @@ def rope_kv_store(q: Optional[Tensor], k: Tensor, v: Tensor, pos_ids: Mapping[st
         q_out = torch.empty((B, H, T, Dh), dtype=q.dtype, device=dev)
     rotate = cos_table is not None
     if rotate:
-        if (cos_table.dtype != torch.float32 or sin_table.dtype != torch.float32
-                or cos_table.shape != sin_table.shape or cos_table.dim() != 2
-                or cos_table.shape[1] != Dh // 2
-                or not cos_table.is_contiguous() or not sin_table.is_contiguous()):
-            raise RuntimeError("cos/sin tables must be contiguous fp32 [rows, Dh/2]")
+        _check_tables(cos_table, sin_table, Dh)
     t_pos, y_pos, x_pos, ps = _pos_triplet(pos_ids, B, T, rotate)
     code = _capi.lib().we_rope_kv_store(
         q.data_ptr() if q is not None else None, k.data_ptr(), v.data_ptr(),
@@ -226,15 +233,8 @@ def rope_kv_attn(q: Tensor, k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor],
     H = q.shape[1]
     if k.dtype != kv.dtype or v.dtype != kv.dtype or q.dtype != kv.dtype:
         raise RuntimeError("q/k/v must have the cache's element type")
-    if kv.dim() != 5 or tuple(kv.shape) != (2, B, Hkv, L + T, Dh) or not kv.is_contiguous():
-        raise RuntimeError("kv must be a contiguous [2, B, Hkv, L+T, Dh] buffer; "
-                           "KV cache expects exactly one frame per upsert")
-    if written.dtype != torch.bool or written.numel() != L + T or not written.is_contiguous():
-        raise RuntimeError("written must be a contiguous bool [L+T] tensor")
-    if (cos_table.dtype != torch.float32 or sin_table.dtype != torch.float32
-            or cos_table.shape != sin_table.shape or cos_table.dim() != 2 or cos_table.shape[1] != Dh // 2
-            or not cos_table.is_contiguous() or not sin_table.is_contiguous()):
-        raise RuntimeError("cos/sin tables must be contiguous fp32 [rows, Dh/2]")
+    _check_cache(kv, written, B, Hkv, T, Dh, L)
+    _check_tables(cos_table, sin_table, Dh)
     t_pos, y_pos, x_pos, ps = _pos_triplet(pos_ids, B, T, True)
     scale = 1.0 / math.sqrt(Dh) if scale is None else float(scale)
     lib = _capi.lib()
