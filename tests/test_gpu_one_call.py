@@ -82,10 +82,12 @@ def test_one_call_outlier_channel(gpu_device):
         assert_attn_close(out, ref, f"t={t}")
 
 
-def test_module_forward_compiles_as_one_graph(gpu_device):
-    """RingAttn under torch.compile(fullgraph=True): the cache call is the registered opaque op
-    (the reference wraps its one native kernel the same way, src/quantize.py:17-42); results and
-    cache state equal the eager module's."""
+@pytest.mark.parametrize("backend,fuse", [("eager", False), ("inductor", False), ("inductor", True)])
+def test_module_forward_compiles_as_one_graph(gpu_device, backend, fuse):
+    """RingAttn under torch.compile(fullgraph=True), also with the backend the reference compiles
+    its passes with (src/world_engine.py:139): the cache call is the registered opaque op (the
+    reference wraps its one native kernel the same way, src/quantize.py:17-42); results and cache
+    state equal the eager module's."""
     import types
     import world_engine_amd as wea
     torch.manual_seed(0)
@@ -94,7 +96,7 @@ def test_module_forward_compiles_as_one_graph(gpu_device):
                                 global_pinned_dilation=1, n_layers=1)
     cos, sin = ro.rope_table_1d(16 * 64, 64)
     rope = wea.RoPE(cos, sin, 8, 8).to(gpu_device)
-    mod = wea.RingAttn(cfg, 0, rope, merged_qkv=True).to(gpu_device, torch.bfloat16)
+    mod = wea.RingAttn(cfg, 0, rope, merged_qkv=True, fuse_elementwise=fuse).to(gpu_device, torch.bfloat16)
     with torch.no_grad():
         mod.gate_proj.weight.normal_(0, 0.5)
     caches = [wea.StaticKVCache(cfg, 1, torch.bfloat16).to(gpu_device) for _ in range(2)]
@@ -102,14 +104,16 @@ def test_module_forward_compiles_as_one_graph(gpu_device):
         c.set_frozen(False)
         for layer in c.layers:
             layer.check_inputs = False
-    compiled = torch.compile(mod, backend="eager", fullgraph=True)
+    compiled = torch.compile(mod, backend=backend, fullgraph=True)
     for t in range(5):
         x = torch.randn(1, 64, 256, device=gpu_device, dtype=torch.bfloat16)
         pos = to_dev(ro.synth_pos_ids(t, 1, 64, 8), gpu_device)
         with torch.no_grad():
             y_e, _ = mod(x, pos, None, caches[0])
             y_c, _ = compiled(x, pos, None, caches[1])
-        assert torch.equal(y_e, y_c), f"t={t}"
+        # the projections around the call may be fused differently by the compiler: tolerance there,
+        # bits for what the library writes
+        assert (y_e.float() - y_c.float()).abs().max().item() <= 2e-2, f"t={t}"
         assert_bits_equal(caches[0].layers[0].kv, caches[1].layers[0].kv, f"cache t={t}")
         assert torch.equal(caches[0].layers[0].written, caches[1].layers[0].written)
 
