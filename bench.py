@@ -71,6 +71,9 @@ def main():
                     help="we_rope_kv_store + we_attn_ring_fwd instead of the one-call we_rope_kv_attn_fwd")
     ap.add_argument("--attn-iters", type=int, default=200, help="attention-only launches for the roofline timing")
     ap.add_argument("--batch", type=int, default=0, help="override the configuration's batch size (experiments)")
+    ap.add_argument("--peaks", action="store_true",
+                    help="also measure what this box reaches on a plain bf16 GEMM (hipBLASLt through torch) and on a "
+                         "streaming copy, and add them to the JSON as measured_peaks")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
                     help="also launch 20 plain copy kernels (read MiB, write MiB each) so a counter run holds "
                          "a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -272,6 +275,33 @@ def main():
                          f"(eager PyTorch CPU, bf16 inputs, fp32 scores), host cpu_count={os.cpu_count()}"}
         log(f"[bench] cpu baseline: {cpu['value']:.0f} us per frame-step on {cpu['cores']} threads")
 
+    peaks = None
+    if args.peaks:
+        # achievable rates on this box next to the published ones the roofline is priced against
+        a = torch.randn(8192, 8192, device=dev, dtype=dtype)
+        b2 = torch.randn(8192, 8192, device=dev, dtype=dtype)
+        src = torch.empty(1 << 28, dtype=torch.int32, device=dev)          # 1 GiB
+        dst = torch.empty_like(src)
+
+        def timed(fn, n):
+            for _ in range(3):
+                fn()
+            torch.cuda.synchronize()
+            s0, s1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s0.record()
+            for _ in range(n):
+                fn()
+            s1.record()
+            torch.cuda.synchronize()
+            return s0.elapsed_time(s1) * 1e-3 / n
+
+        t_mm = timed(lambda: torch.matmul(a, b2), 20)
+        t_cp = timed(lambda: torch.add(src, 0, out=dst), 20)
+        peaks = {"bf16_gemm_8192_tflops": round(2 * 8192 ** 3 / t_mm / 1e12, 1),
+                 "copy_1gib_read_plus_write_gbps": round(2 * src.numel() * 4 / t_cp / 1e9, 1)}
+        log(f"[bench] measured on this box: {peaks}")
+        del a, b2, src, dst
+
     result = {
         "metric": "attn_us_per_frame_step",
         "value": round(ms_per_step * 1e3, 3),
@@ -294,6 +324,8 @@ def main():
         "roofline": roof,
         "cpu_baseline": cpu,
     }
+    if peaks is not None:
+        result["measured_peaks"] = peaks
     print(json.dumps(result), flush=True)
 
 
