@@ -316,7 +316,8 @@ def main():
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": c["name"], "launch": "eager" if args.eager else "hip_graph",
-                   "calls_per_step": f"{layers} x (we_rope_kv_store + we_attn_ring_fwd)",
+                   "calls_per_step": f"{layers} x " + ("(we_rope_kv_store + we_attn_ring_fwd)" if args.two_calls
+                                                       else "we_rope_kv_attn_fwd (store kernel + attention kernels)"),
                    "n_splits": n_splits, "q_tile": args.q_tile or "auto"},
         "us_per_layer_step": round(us_per_layer_step, 3),
         "attn_tflops": round(tflops, 2),
