@@ -382,7 +382,8 @@ attn_ring_kernel(AttnParams p) {
   };
   // nkeys: keys that exist in the block whose logits this step computes (32 = all, 0 = the block
   // lies past the end of the split)
-  auto step = [&](auto koff_c, auto voff_c, auto nkoff_c, auto nvoff_c, int nkeys, auto&& mid) __attribute__((always_inline)) {
+  // (the K fragments at koff_c were requested by the previous step; the offset documents the call)
+  auto step = [&](auto /*koff_c*/, auto voff_c, auto nkoff_c, auto nvoff_c, int nkeys, auto&& mid) __attribute__((always_inline)) {
     const bool live = nkeys > 0;
     if (pending) {
 #pragma unroll
@@ -392,8 +393,8 @@ attn_ring_kernel(AttnParams p) {
     }
     pending = false;
 
-    // reads issued since this step's read 0 / next own V fragment / next-step read pairs issued
-    int issued = PRE, vnext = 1, npair = 0;
+    // next own V fragment to request / next-step read pairs requested so far
+    int vnext = 1, npair = 0;
     constexpr int NPAIR = PRE / 2;            // the next step's first reads go out two at a time
     constexpr int I0 = NV - 1 - NPAIR;        // ... after the product MFMAs I0, I0+1, ...
     auto next_pair = [&]() __attribute__((always_inline)) {
@@ -404,7 +405,6 @@ attn_ring_kernel(AttnParams p) {
         read_v(nvoff_c, 0);
       }
       ++npair;
-      issued += 2;
     };
 
     // From here to the end of the product the issue order is pinned statement by statement
@@ -434,8 +434,7 @@ attn_ring_kernel(AttnParams p) {
       if (vnext < NV && ks <= 12 - KS) {
         read_v(voff_c, vnext);
         ++vnext;
-        issued += 2;
-      }
+        }
       exp_slot(1 + ks);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -446,8 +445,7 @@ attn_ring_kernel(AttnParams p) {
       if (vnext < NV) {  // reads 0..KS+2i-1 have completed: room for one more fragment
         read_v(voff_c, vnext);
         ++vnext;
-        issued += 2;
-      }
+        }
       typedef unsigned int u32x4v __attribute__((ext_vector_type(4)));
       const u32x4v a4 = __builtin_shufflevector(v0[i], v1[i], 0, 1, 2, 3);
       o[i % DB] = M::mma(__builtin_bit_cast(frag_t, a4), p_prev[i / DB], o[i % DB]);
