@@ -209,3 +209,38 @@ def test_attention_kernels_keep_their_state_in_registers():
     sizes = [int(m) for m in re.findall(r"ScratchSize \[bytes/lane\]: (\d+)", r.stderr)]
     assert len(sizes) == 16, sizes          # bf16/f16 x Dh 64/128 x 128/256 queries x ragged or not
     assert max(sizes) <= 160, sizes
+
+
+def test_three_axis_rope_table_structure():
+    """What the geometry fixes about the three-axis table (the per-axis spectra themselves come
+    from a package that is not available here, so their values stay unpinned): block widths, which
+    coordinate each block depends on, doubled frequencies, mirror symmetry of the pixel axes,
+    angles below Nyquist, a unit first temporal frequency; and the oracle's restatement agrees."""
+    from oracle import ring_oracle as ro
+    Hh, Ww, n_frames, Dh = 6, 10, 5, 64
+    rope = wea.RoPE.three_axis(n_frames, Dh, Hh, Ww)
+    assert rope.cos.shape == rope.sin.shape == (n_frames * Hh * Ww, Dh // 2) and rope.cos.dtype == torch.float32
+    ang = torch.atan2(rope.sin, rope.cos).view(n_frames, Hh, Ww, Dh // 2)
+    bx, by = slice(0, Dh // 8), slice(Dh // 8, Dh // 4)
+    bt = slice(Dh // 4, Dh // 2)
+    cos = rope.cos.view(n_frames, Hh, Ww, -1)
+    sin = rope.sin.view(n_frames, Hh, Ww, -1)
+    # X depends on x only, Y on y only, T on t only
+    assert torch.equal(cos[..., bx], cos[:1, :1, :, bx].expand(n_frames, Hh, Ww, -1))
+    assert torch.equal(cos[..., by], cos[:1, :, :1, by].expand(n_frames, Hh, Ww, -1))
+    assert torch.equal(sin[..., bt], sin[:, :1, :1, bt].expand(n_frames, Hh, Ww, -1))
+    # each frequency appears twice in a row
+    assert torch.equal(cos[..., 0::2], cos[..., 1::2]) and torch.equal(sin[..., 0::2], sin[..., 1::2])
+    # pixel positions are symmetric about the centre: angle(x) = -angle(W-1-x)
+    assert torch.allclose(cos[..., bx], cos[..., bx].flip(2), atol=1e-6)
+    assert torch.allclose(sin[..., bx], -sin[..., bx].flip(2), atol=1e-6)
+    assert torch.allclose(sin[..., by], -sin[..., by].flip(1), atol=1e-6)
+    # neighbouring pixels differ by less than pi in every column (below Nyquist), and by more than 0
+    step_x = (ang[0, 0, 1, bx] - ang[0, 0, 0, bx]).remainder(2 * torch.pi)
+    assert (step_x > 0).all() and (step_x < torch.pi).all()
+    # frame 0 is the identity rotation on the temporal block; the first temporal frequency is 1 rad/frame
+    assert torch.equal(cos[0, ..., bt], torch.ones_like(cos[0, ..., bt])) and not sin[0, ..., bt].any()
+    assert torch.allclose(ang[1, 0, 0, bt][0], torch.tensor(1.0), atol=1e-6)
+    assert (ang[1, 0, 0, bt][0::2].diff() < 0).all()      # geometric spectrum: decreasing
+    o_cos, o_sin = ro.ortho_rope_table(Hh, Ww, n_frames, Dh)
+    assert torch.allclose(rope.cos, o_cos, atol=1e-6) and torch.allclose(rope.sin, o_sin, atol=1e-6)

@@ -50,6 +50,36 @@ class RoPE(nn.Module):
         ang = torch.arange(n_rows, dtype=torch.float64)[:, None] * inv[None, :]
         return cls(ang.cos().float(), ang.sin().float(), height, width)
 
+    @classmethod
+    def three_axis(cls, n_frames: int, d_head: int, height: int, width: int):
+        """Table of the reference's ``OrthoRoPE`` (``src/model/attn.py:46-67``): angle columns
+        ``[X | Y | T]`` of ``Dh/8 + Dh/8 + Dh/4``, rows ordered ``(t, y, x)``.  X and Y use a linear
+        "pixel" spectrum over positions ``linspace(-1 + 1/n, 1 - 1/n, n)`` with top frequency
+        ``0.8 * min(height, width)``; T uses the geometric "lang" spectrum over the frame index.
+
+        The per-axis spectra are those of ``rotary_embedding_torch`` (>= 0.8.8 per the reference's
+        ``pyproject.toml:14``), a package that is not available offline: 'pixel' is
+        ``linspace(1, max_freq/2, dim/2) * pi``, 'lang' is ``10000**(-2i/dim)``, each frequency
+        taken twice in a row.  These formulas are restated from the package's published source and
+        have not been checked against it here; the kernels consume any table, so only positions of
+        real checkpoints depend on this builder."""
+        if d_head % 16 != 0:
+            raise AssertionError("d_head must be a multiple of 16 for the three-axis table")
+        dim_xy, dim_t = d_head // 8, d_head // 4
+        pixel = torch.linspace(1.0, min(height, width) * 0.8 / 2, dim_xy // 2) * math.pi
+        lang = 1.0 / (10000.0 ** (torch.arange(0, dim_t, 2)[: dim_t // 2].float() / dim_t))
+        x_pos = torch.linspace(-1 + 1 / width, 1 - 1 / width, width)
+        y_pos = torch.linspace(-1 + 1 / height, 1 - 1 / height, height)
+        ang_x = (x_pos[:, None] * pixel[None, :]).repeat_interleave(2, dim=-1)              # [W, Dh/8]
+        ang_y = (y_pos[:, None] * pixel[None, :]).repeat_interleave(2, dim=-1)              # [H, Dh/8]
+        ang_t = (torch.arange(n_frames).float()[:, None] * lang[None, :]).repeat_interleave(2, dim=-1)
+        table = torch.cat([
+            ang_x[None, None, :, :].expand(n_frames, height, width, -1),
+            ang_y[None, :, None, :].expand(n_frames, height, width, -1),
+            ang_t[:, None, None, :].expand(n_frames, height, width, -1),
+        ], dim=-1).reshape(n_frames * height * width, d_head // 2)
+        return cls(table.cos(), table.sin(), height, width)
+
     def forward(self, x: Tensor, pos_ids: Mapping[str, Tensor]) -> Tensor:
         return ops.rope_apply(x, pos_ids, self.cos, self.sin, self.height, self.width)
 
