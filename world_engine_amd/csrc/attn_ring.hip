@@ -76,7 +76,7 @@ __device__ __forceinline__ void dma16(uint64_t gbase, uint32_t voff, uint32_t ld
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                :
                : "v"(voff), "s"(gbase), "s"(lds_addr)
-               : "memory");
+               : "memory", "m0");
 }
 template <int N>
 __device__ __forceinline__ void dma_wait() {
