@@ -713,13 +713,18 @@ attn_ring_kernel(AttnParams p) {
 
 template <typename M, int DH, int KSPLIT, bool RAGGED>
 static hipError_t launch_ring_r(const AttnParams& p, hipStream_t stream) {
-  static bool configured = false;
+  // the LDS limit of a kernel is a per-device setting: raise it once on every device that launches
+  // (a flag that two threads both find unset is set twice, which is harmless)
+  static bool configured[64] = {};
   const int lds = RingLds<DH>::kBytes;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_ring_kernel<M, DH, KSPLIT, RAGGED>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= 64 || !configured[dev]) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_ring_kernel<M, DH, KSPLIT, RAGGED>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
-    configured = true;
+    if (dev >= 0 && dev < 64) configured[dev] = true;
   }
   const int rounds = (p.unit_splits + 7) / 8;
   const dim3 grid((unsigned)(8 * p.q_tiles), (unsigned)p.group, (unsigned)rounds);
