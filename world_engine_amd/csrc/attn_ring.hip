@@ -352,8 +352,6 @@ attn_ring_kernel(AttnParams p) {
   //   VALU:         the probabilities of the current block (s_cur -> p_cur).
   // LDS reads are issued in consumption order - K fragments 0..KS-1, then the NV V^T fragments
   // (two transposing reads each) - running up to 15 reads ahead of the MFMAs.
-  bool pending = false;   // an accumulator rescale decided in the previous step is due
-  float alpha = 1.f;
   frag_t p_prev[2];
   f32x16_t s_cur;
   // Fragment registers live across steps: every step starts with its first PRE reads (all K
@@ -384,15 +382,8 @@ attn_ring_kernel(AttnParams p) {
   // lies past the end of the split)
   // (the K fragments at koff_c were requested by the previous step; the offset documents the call)
   auto step = [&](auto /*koff_c*/, auto voff_c, auto nkoff_c, auto nvoff_c, int nkeys, auto&& mid) __attribute__((always_inline)) {
-    const bool live = nkeys > 0;
-    if (pending) {
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
-    }
-    pending = false;
-
+    // logits of a block past the end are never consumed; only a short tile's empty block needs them dead
+    const bool live = !RAGGED || nkeys > 0;
     // next own V fragment to request / next-step read pairs requested so far
     int vnext = 1, npair = 0;
     constexpr int NPAIR = PRE / 2;            // the next step's first reads go out two at a time
@@ -465,19 +456,23 @@ attn_ring_kernel(AttnParams p) {
 
     if (__ballot(!(rs <= 256.f)) != 0ull) {
       // Rare: some probability of this block may exceed 2^8.  Raise the reference of the rows
-      // that need it, redo the block's probabilities exactly, and re-base the logits of the next
-      // block, which were produced with the old reference.
+      // that need it, redo the block's probabilities exactly, re-base the logits of the next
+      // block, which were produced with the old reference, and rescale the accumulators: they hold
+      // the blocks before this one (the last of those products was issued above).
       const float mx = block_max(s_cur);
       const float m_new = mx > 0.f ? M::round_up(m_ref + mx) : m_ref;
       const float delta = m_new - m_ref;
-      alpha = __builtin_amdgcn_exp2f(-delta);
+      const float alpha = __builtin_amdgcn_exp2f(-delta);
       rs = probabilities(p_cur, s_cur, delta);
       l_run *= alpha;
       m_ref = m_new;
       set_shift();
 #pragma unroll
       for (int i = 0; i < 16; ++i) s_next[i] -= delta;
-      pending = true;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
     }
     l_run += rs;
     p_prev[0] = p_cur[0];
@@ -603,12 +598,6 @@ attn_ring_kernel(AttnParams p) {
     if (j < ntile) { iteration(j, IntC<2>()); ++j; }
 
     // product of the last block: (ntile-1, 1) for full-tile wavefronts, (ntile-1, hb) otherwise
-    if (pending) {
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
-    }
     {
       const int last = (ntile - 1) % NST;
       const unsigned char* vt = smem + v_rd + last * TILE_B + (KSPLIT == 1 ? KB_B : 0);
