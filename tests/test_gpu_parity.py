@@ -194,6 +194,19 @@ def test_attention_fp32_ragged_frame(gpu_device):
         assert (p.attend(q_h, ring).cpu() - ro.attention_fp32(q_o, k_all, v_all, mask)).abs().max().item() <= 1e-5
 
 
+@pytest.mark.parametrize("n_slots,T,Dh,kw", [(80, 64, 64, {"n_splits": 1}), (130, 64, 128, {}),
+                                             (70, 96, 64, {"n_splits": 2, "q_tile": 256})])
+def test_attention_rings_longer_than_one_wavefront(gpu_device, n_slots, T, Dh, kw):
+    """More ring slots than a wavefront has lanes, and more tiles per workgroup than one batch of
+    precomputed tile offsets holds: the slot list spans several rounds and the offsets are
+    reloaded inside the tile loop.  Runs until the ring has wrapped."""
+    _say(f"long ring n_slots={n_slots} T={T} Dh={Dh} {kw}")
+    p = Pair(gpu_device, torch.bfloat16, B=1, H=2, Hkv=1, T=T, Dh=Dh, n_slots=n_slots, cfg_id=53,
+             table_rows=(n_slots + 12) * T)
+    steps = n_slots + 8
+    _run_and_check(p, steps, check_steps={0, 1, 63, 64, 65, 66, n_slots - 1, n_slots, n_slots + 1, steps - 1}, **kw)
+
+
 def test_attention_partial_round_tail_split(gpu_device):
     """320 workgroups = one full round of 256 CUs plus a quarter round: the library splits the
     context of the last 32 heads only (mixed direct-output and workspace rows in one call)."""

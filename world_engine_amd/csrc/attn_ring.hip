@@ -174,8 +174,7 @@ attn_ring_kernel(AttnParams p) {
 
   // ---- list of visible slots (the tail is pseudo-slot n_slots) ----
   // Every wavefront builds it for itself (no barrier, no serial section) in a private strip of
-  // LDS: lane i of round k looks at slot 64*k + i.  Entries 0..63 then live in one register (lane
-  // i holds entry i), which is where the hot loop looks them up; longer lists fall back to LDS.
+  // LDS: lane i of round k looks at slot 64*k + i.
   int* vis = reinterpret_cast<int*>(smem + L::MISC_OFF) + wave * (WE_MAX_SLOTS + 64);
   int nvis = 0;
   {
@@ -191,11 +190,6 @@ attn_ring_kernel(AttnParams p) {
     if (lane == 0) vis[nvis] = p.n_slots;
     ++nvis;
   }
-  const int vis0 = lane < nvis ? vis[lane] : 0;
-  auto vis_at = [&](int i) __attribute__((always_inline)) {
-    if (__builtin_expect(i < 64, 1)) return __builtin_amdgcn_readlane(vis0, i);
-    return __builtin_amdgcn_readfirstlane(vis[i]);
-  };
   // tiles per slot; the last one of a slot holds t_last of its 64 keys when T % 64 != 0
   const int tps = (p.T + BN - 1) / BN;
   const int t_last = p.T - (tps - 1) * BN;
@@ -222,53 +216,48 @@ attn_ring_kernel(AttnParams p) {
     kvoff[i] = row * ROW_B + ((phys ^ k_swz<DH>(row)) << 4);
     vvoff[i] = row * ROW_B + ((phys ^ v_swz<DH>(row)) << 4);
   }
-  struct TileWalk {  // position of a load stream in the split's list of visible tiles
-    int sidx, sub, left;
+  // The split's visible tiles, 64 at a time: lane i of toff holds the byte offset, inside the
+  // (batch, kv head) plane, of tile 64*k + i of the split (fits 32 bits, checked on the host).
+  // Bit 0 (row starts are multiples of 128 bytes) marks the short last tile of a slot.  The tile
+  // loop then needs one v_readlane per tile instead of walking slots and tiles with scalar code.
+  uint32_t toff = 0;
+  auto load_offsets = [&](int first) __attribute__((always_inline)) {
+    unsigned ti = (unsigned)(t_begin + first + lane);
+    if (ti > (unsigned)(t_end - 1)) ti = (unsigned)(t_end - 1);
+    const unsigned sidx = ti / (unsigned)tps;
+    const unsigned sub = ti - sidx * (unsigned)tps;
+    const uint32_t o = ((uint32_t)vis[sidx] * (uint32_t)p.T + sub * BN) * (uint32_t)ROW_B;
+    toff = (ragged && sub == (unsigned)(tps - 1)) ? (o | 1u) : o;
   };
-  auto walk_init = [&]() __attribute__((always_inline)) {
-    TileWalk w;
-    w.sidx = t_begin / tps;
-    w.sub = t_begin - w.sidx * tps;
-    w.left = ntile - 1;
-    return w;
-  };
-  auto walk_next = [&](TileWalk& w) __attribute__((always_inline)) {  // stays on the last tile
-    if (w.left > 0) {
-      --w.left;
-      if (++w.sub == tps) {
-        w.sub = 0;
-        ++w.sidx;
-      }
-    }
-  };
-  // byte offset of a tile inside its (batch, kv head) plane; fits 32 bits (checked on the host).
-  // Bit 0 (row starts are multiples of 128 bytes) marks the short last tile of a slot.
-  auto tile_off = [&](const TileWalk& w) __attribute__((always_inline)) {
-    const uint32_t o = (uint32_t)(vis_at(w.sidx) * p.T + w.sub * BN) * (uint32_t)ROW_B;
-    return (ragged && w.sub == tps - 1) ? (o | 1u) : o;
+  int kc = 0;  // tile the K stream requests next; it stays on the last one
+  auto next_off = [&]() __attribute__((always_inline)) {
+    if ((kc & 63) == 0) load_offsets(kc);
+    const uint32_t o = (uint32_t)__builtin_amdgcn_readlane((int)toff, kc & 63);
+    if (kc < ntile - 1) ++kc;
+    return o;
   };
   const uint64_t kplane = uniform64(kbase), vplane = uniform64(vbase);
+  const uint32_t wave_lds = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + wave * 1024));
   // A short tile must not read rows of the next slot (or past the end of the buffer): its rows
   // beyond t_last repeat row t_last - 1; their keys are masked out of the softmax further down.
   auto clamp_rows = [&](uint32_t voff, int i) __attribute__((always_inline)) {
     const int row = (wave + i * 8) * RPI + lane / CPR;
     return row < t_last ? voff : voff - (uint32_t)(row - (t_last - 1)) * ROW_B;
   };
+  // the tile offset is uniform: it goes into the scalar base address, not into every lane's offset
   auto dma_k = [&](uint32_t off, int slot) __attribute__((always_inline)) {
-    const bool cut = (off & 1u) != 0u;
-    off &= ~1u;
+    const bool cut = RAGGED && (off & 1u) != 0u;
+    const uint64_t base = kplane + (off & ~1u);
 #pragma unroll
     for (int i = 0; i < NDMA; ++i)
-      dma16(kplane, (cut ? clamp_rows(kvoff[i], i) : kvoff[i]) + off,
-            __builtin_amdgcn_readfirstlane(lds0 + slot * TILE_B + (wave + i * 8) * 1024));
+      dma16(base, cut ? clamp_rows(kvoff[i], i) : kvoff[i], wave_lds + slot * TILE_B + i * 8 * 1024);
   };
   auto dma_v = [&](uint32_t off, int slot) __attribute__((always_inline)) {
-    const bool cut = (off & 1u) != 0u;
-    off &= ~1u;
+    const bool cut = RAGGED && (off & 1u) != 0u;
+    const uint64_t base = vplane + (off & ~1u);
 #pragma unroll
     for (int i = 0; i < NDMA; ++i)
-      dma16(vplane, (cut ? clamp_rows(vvoff[i], i) : vvoff[i]) + off,
-            __builtin_amdgcn_readfirstlane(lds0 + L::V_OFF + slot * TILE_B + (wave + i * 8) * 1024));
+      dma16(base, cut ? clamp_rows(vvoff[i], i) : vvoff[i], wave_lds + L::V_OFF + slot * TILE_B + i * 8 * 1024);
   };
   // keys of 32-key block blk of the tile at position sub of its slot that exist (0 .. 32)
   auto block_keys = [&](int sub, int blk) __attribute__((always_inline)) {
@@ -414,7 +403,12 @@ attn_ring_kernel(AttnParams p) {
     auto exp_slot = [&](int g) __attribute__((always_inline)) {
 #pragma unroll
       for (int t = 0; t < EPS; ++t)
-        if (g * EPS + t < 16) e[g * EPS + t] = __builtin_amdgcn_exp2f(s_cur[g * EPS + t]);
+        if (g * EPS + t < 16) {
+          e[g * EPS + t] = __builtin_amdgcn_exp2f(s_cur[g * EPS + t]);
+          // an exponential has no side effect, so nothing else keeps it in its slot: left alone the
+          // compiler sinks the first nine of a step below the tile DMAs
+          asm volatile("" : "+v"(e[g * EPS + t]));
+        }
     };
     exp_slot(0);
     __builtin_amdgcn_sched_barrier(0);
@@ -495,17 +489,16 @@ attn_ring_kernel(AttnParams p) {
     // what the iterations before 0 would have.
     constexpr int KA = KSPLIT == 1 ? 3 : 4;
     // The V stream trails the K stream by KA - 2 tiles, so it reuses the K stream's offsets.
-    TileWalk kw = walk_init();
-    int csub = kw.sub;  // position in its slot of the tile whose logits are computed next
+    int csub = t_begin - (t_begin / tps) * tps;  // position in its slot of the tile whose logits are computed next
     uint32_t off1, off2;  // offsets of the last and the last-but-one tile the K stream visited
     // Q was requested before the slot flags and loads return in order, so it is here; stating a
     // use now keeps the wait for it from landing behind the tile DMAs issued next.
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) asm volatile("" ::"v"(qf[ks]));
     {
-      const uint32_t o0 = tile_off(kw); walk_next(kw);
-      const uint32_t o1 = tile_off(kw); walk_next(kw);
-      const uint32_t o2 = tile_off(kw); walk_next(kw);
+      const uint32_t o0 = next_off();
+      const uint32_t o1 = next_off();
+      const uint32_t o2 = next_off();
       dma_k(o0, 0);
       dma_k(o1, 1);
       if (KSPLIT == 2) dma_k(o2, 2);
@@ -514,7 +507,7 @@ attn_ring_kernel(AttnParams p) {
         dma_k(o2, 2);
         off1 = o2; off2 = o1;
       } else {
-        const uint32_t o3 = tile_off(kw); walk_next(kw);
+        const uint32_t o3 = next_off();
         dma_k(o3, 3);
         off1 = o3; off2 = o2;
       }
@@ -557,8 +550,7 @@ attn_ring_kernel(AttnParams p) {
     auto iteration = [&](int j, auto jm_c) __attribute__((always_inline)) {
       constexpr int JM = decltype(jm_c)::value;
       auto issue_dma = [&]() __attribute__((always_inline)) {
-        const uint32_t o = tile_off(kw);
-        walk_next(kw);
+        const uint32_t o = next_off();
         dma_k(o, (JM + KA) % NST);                       // K(j+KA)
         dma_v(KA == 3 ? off1 : off2, (JM + 2) % NST);    // V(j+2)
         off2 = off1;
