@@ -575,7 +575,13 @@ attn_ring_kernel(AttnParams p) {
       }
       csub = nsub;
       dma_wait<2 * NDMA>();  // all but this iteration's two tiles have landed (this wavefront's part)
-      __syncthreads();
+      // A bare barrier: __syncthreads() would also wait for every LDS read in flight, i.e. for the
+      // next step's fragments requested a moment ago.  Nothing needs that: the tiles arrive by DMA,
+      // whose completion the counter wait above tracks, fragment reads are awaited where they are
+      // used, and the reads still in flight here target ring slots that no DMA overwrites before
+      // the barrier after next.  The empty asm keeps the compiler from moving memory accesses across.
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
     };
 
     int j = 0;
