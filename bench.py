@@ -31,7 +31,7 @@ PEAK_BF16_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
 # two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) with the library's own split/tile choice, each
 # scaled by the same counter's reading for a 256 MiB copy kernel (FETCH_SIZE x2.000, WRITE_SIZE
 # x1.000); the summaries are profiles/attn_ring_cfg{1,3}_hbm_traffic.txt.
-MEASURED_TRAFFIC = {1: 60657944, 3: 496852454}
+MEASURED_TRAFFIC = {1: 60658972, 3: 496861378}
 
 CONFIGS = {
     1: dict(name="cfg1: B=1 H=16 Dh=128 T=256 16-slot ring (4096-token context) bf16, steady-state wrap",
