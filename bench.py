@@ -263,7 +263,7 @@ def main():
         done, spent = 0, 0.0
         budget = 12.0 if c["B"] * c["H"] * c["T"] <= 16 * 256 else 20.0
         ro.layer_step(oc, 0, q, k, v, ro.synth_pos_ids(n, B, T, W), cos, sin, T // W, W)   # untimed warm-up
-        while spent < budget and done < 50:
+        while spent < budget and done < 1000:    # about 12 s of host work (20 s for the large shapes)
             pos_c = ro.synth_pos_ids(n + 1 + done, B, T, W)
             t0c = time.perf_counter()
             ro.layer_step(oc, 0, q, k, v, pos_c, cos, sin, T // W, W)
