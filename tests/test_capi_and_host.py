@@ -244,3 +244,41 @@ def test_three_axis_rope_table_structure():
     assert (ang[1, 0, 0, bt][0::2].diff() < 0).all()      # geometric spectrum: decreasing
     o_cos, o_sin = ro.ortho_rope_table(Hh, Ww, n_frames, Dh)
     assert torch.allclose(rope.cos, o_cos, atol=1e-6) and torch.allclose(rope.sin, o_sin, atol=1e-6)
+
+
+def test_header_is_plain_c_and_links_against_the_library(tmp_path):
+    """The boundary is a C ABI: the header must compile as C99 on its own, and a C program that
+    includes it must link against the built library and get the documented status codes back
+    from calls that are rejected before anything touches a GPU."""
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no C compiler")
+    lib_path = _capi.library_path() if hasattr(_capi, "library_path") else os.path.join(ROOT, "world_engine_amd", "libwe_attn.so")
+    src = tmp_path / "abi.c"
+    src.write_text(r'''
+#include "we_attn.h"
+#include <stdio.h>
+int main(void) {
+  int64_t s[3] = {8, 8, 8};
+  /* NULL pointers are refused first */
+  int rc_null = we_attn_ring_fwd(0, s, 0, 0, 0, 0, s, 0, 0, 1, 1, 1, 64, 64, 128, 1, 0.125f, 0, 0, WE_DTYPE_BF16, 0);
+  size_t ws = we_attn_workspace_bytes(1, 16, 16, 256, 128, 4096, 4, 0);
+  printf("%d %d %zu %s\n", we_version(), rc_null, ws, we_error_string(WE_ERR_WORKSPACE));
+  return 0;
+}
+''')
+    exe = tmp_path / "abi"
+    r = subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", f"-I{os.path.join(ROOT, 'include')}",
+                        str(src), "-o", str(exe), lib_path, f"-Wl,-rpath,{os.path.dirname(lib_path)}",
+                        "-Wl,-rpath,/opt/rocm/lib", "-Wl,--allow-shlib-undefined"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-3000:]
+    out = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert out.returncode == 0, out.stderr[-2000:]
+    version, rc_null, ws, msg = out.stdout.strip().split(" ", 3)
+    lib = _capi.lib()
+    assert int(version) == lib.we_version()
+    assert int(rc_null) == -1                                    # WE_ERR_NULL_POINTER
+    assert int(ws) == 4 * 16 * 256 * (128 * 2 + 8)
+    assert "workspace" in msg
