@@ -1,15 +1,23 @@
 #!/usr/bin/env python3
 """Benchmark of the frame-causal ring-buffer attention hot path on one MI355X.
 
-A *step* is one frame-step of one attention layer: the fused RoPE + ring-slot K/V store followed
-by the attention over the ring (one we_rope_kv_store call + one we_attn_ring_fwd call through the
-C ABI).  The default workload is benchmark configuration 1 (B=1, H=16, Dh=128, 256 tokens per frame,
-16-slot ring, bf16); ``--config 2|3|4`` select the other single-GPU configurations.  Inputs are
-synthetic N(0,1) tensors already resident in HBM, laid out like the merged QKV projection output.
-The timed region replays a HIP graph holding exactly K consecutive steps (the ring advances every
-step, as in the real schedule), bracketed by device synchronisation.
+A *step* is one attention call of the frame schedule for every layer of a configuration: the
+fused RoPE + ring-slot K/V store followed by the attention over the ring (we_rope_kv_attn_fwd
+through the C ABI).  The default run measures benchmark configurations 1-4 one after the other
+and prints ONE JSON line: its top level is configuration 1 (B=1, H=16, Dh=128, 256 tokens per
+frame, 16-slot ring, bf16; the configuration the metric is quoted on) and ``configs`` holds the
+same figures for every configuration, among them the two the targets are stated on: cfg3
+(1024-token frames, MFMA-bound) and cfg4 (256-token frames at 8K context, HBM-bound).
+``--config N`` measures only configuration N (profiling runs).
 
-Prints ONE JSON line on stdout; progress goes to stderr.
+Inputs are synthetic N(0,1) tensors already resident in HBM, laid out like the merged QKV
+projection output.  The timed region replays a HIP graph holding exactly K consecutive steps (the
+ring advances every step, as in the real schedule) back to back until it lasts at least 5 ms,
+bracketed by device synchronisation; it is sampled several times and the median is reported with
+the 10th and 90th percentile beside it.
+
+Progress goes to stderr.  The JSON line is printed even when the CPU leg fails (the process then
+still exits non-zero).
 """
 from __future__ import annotations
 
@@ -17,8 +25,10 @@ import argparse
 import json
 import math
 import os
+import re
 import sys
 import time
+import traceback
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
@@ -26,23 +36,21 @@ if ROOT not in sys.path:
 
 PEAK_HBM_GBPS = 8000.0       # MI355X HBM3E, published
 PEAK_BF16_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
-
-# HBM-side bytes per attention call (attn_ring_kernel + attn_combine_kernel, reads + writes) from
-# two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) with the library's own split/tile choice, each
-# scaled by the same counter's reading for a 256 MiB copy kernel (FETCH_SIZE x2.000, WRITE_SIZE
-# x1.000); the summaries are profiles/attn_ring_cfg{1,3}_hbm_traffic.txt.
-MEASURED_TRAFFIC = {1: 60658972, 3: 496861378}
+MIN_REGION_S = 5e-3          # a timing sample lasts at least this long
+SAMPLES = 9                  # timing samples per figure (median, p10, p90)
 
 CONFIGS = {
     1: dict(name="cfg1: B=1 H=16 Dh=128 T=256 16-slot ring (4096-token context) bf16, steady-state wrap",
-            B=1, H=16, Hkv=16, Dh=128, T=256, slots=16, layers=1, frozen_subs=0, bound="hbm"),
+            B=1, H=16, Hkv=16, Dh=128, T=256, slots=16, layers=1, frozen_subs=0, bound="hbm", cpu_budget_s=8.0),
     2: dict(name="cfg2: 24 layers x cfg1 shapes, own ring per layer, K outlier channel",
-            B=1, H=16, Hkv=16, Dh=128, T=256, slots=16, layers=24, frozen_subs=0, bound="hbm", outlier=True),
+            B=1, H=16, Hkv=16, Dh=128, T=256, slots=16, layers=24, frozen_subs=0, bound="hbm", outlier=True,
+            cpu_budget_s=6.0),
     3: dict(name="cfg3: B=4 H=24 Dh=128 T=1024 8-slot ring (8192-token context) bf16",
-            B=4, H=24, Hkv=24, Dh=128, T=1024, slots=8, layers=1, frozen_subs=0, bound="mfma"),
-    4: dict(name="cfg4: B=1 H=16 Dh=128 T=256 32-slot ring, 4 frozen substeps + 1 persisting call per frame",
-            B=1, H=16, Hkv=16, Dh=128, T=256, slots=32, layers=1, frozen_subs=4, bound="hbm"),
+            B=4, H=24, Hkv=24, Dh=128, T=1024, slots=8, layers=1, frozen_subs=0, bound="mfma", cpu_budget_s=10.0),
+    4: dict(name="cfg4: B=1 H=16 Dh=128 T=256 32-slot ring (8192-token context), 4 frozen substeps + 1 persisting call per frame",
+            B=1, H=16, Hkv=16, Dh=128, T=256, slots=32, layers=1, frozen_subs=4, bound="hbm", cpu_budget_s=6.0),
 }
+HEADLINE = 1
 
 
 def log(*a):
@@ -57,68 +65,93 @@ def algorithmic_work(c, n_vis):
     return flops, byts
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=512)
-    ap.add_argument("--warmup", type=int, default=32)
-    ap.add_argument("--config", type=int, default=1, choices=sorted(CONFIGS))
-    ap.add_argument("--n-splits", type=int, default=0, help="context splits (0 = library's choice)")
-    ap.add_argument("--q-tile", type=int, default=0, help="queries per workgroup (0 = library's choice)")
-    ap.add_argument("--eager", action="store_true", help="launch from Python per call instead of a HIP graph")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--two-calls", action="store_true",
-                    help="we_rope_kv_store + we_attn_ring_fwd instead of the one-call we_rope_kv_attn_fwd")
-    ap.add_argument("--attn-iters", type=int, default=200, help="attention-only launches for the roofline timing")
-    ap.add_argument("--batch", type=int, default=0, help="override the configuration's batch size (experiments)")
-    ap.add_argument("--peaks", action="store_true",
-                    help="also measure what this box reaches on a plain bf16 GEMM (hipBLASLt through torch) and on a "
-                         "streaming copy, and add them to the JSON as measured_peaks")
-    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
-                    help="also launch 20 plain copy kernels (read MiB, write MiB each) so a counter run holds "
-                         "a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
-    args = ap.parse_args()
+def schedule_plan(c, steps, warmup, cpu_window=8):
+    """Frame arithmetic of one configuration's run, in one place so that it can be checked without
+    a GPU.  Step s of the schedule belongs to frame s // subs (subs = attention calls per frame).
+    Untimed ring fill = slots * subs steps, then `warmup` steps, then `steps` timed steps; the
+    attention-only leg uses one further frame; the CPU leg cycles over `cpu_window` frames after
+    that.  `table_frames` is how many frames the RoPE table must cover (every frame index any leg
+    uses is below it)."""
+    subs = c["frozen_subs"] + 1
+    fill_steps = c["slots"] * subs
+    first = fill_steps + warmup
+    last_timed_frame = (first + steps - 1) // subs
+    attn_frame = last_timed_frame + 1
+    cpu_first = attn_frame + 1
+    cpu_frames = [cpu_first + i for i in range(cpu_window)]
+    table_frames = cpu_frames[-1] + 1
+    return dict(subs=subs, fill_steps=fill_steps, first=first, last_timed_frame=last_timed_frame,
+                attn_frame=attn_frame, cpu_frames=cpu_frames, table_frames=table_frames)
 
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py measures the single-GPU hot path only: this build has no multi-GPU path "
-              "(heads and batch streams would shard with no communication); run with --gpus 1.",
-              file=sys.stderr)
-        sys.exit(2)
 
-    import torch
-    from oracle import ring_oracle as ro           # inputs + the cpu_baseline leg only
-    import world_engine_amd as wea
-    from world_engine_amd import ops
+def max_table_row(frame, T):
+    """Largest RoPE-table row a frame touches (row = t*T + token for the 1-D table of the configurations)."""
+    return frame * T + T - 1
 
-    c = dict(CONFIGS[args.config])
-    if args.batch:
-        c["B"] = args.batch
-        c["name"] += f" [batch overridden to {args.batch}]"
+
+def percentile(xs, p):
+    xs = sorted(xs)
+    if len(xs) == 1:
+        return xs[0]
+    pos = p * (len(xs) - 1)
+    lo = int(math.floor(pos))
+    hi = min(lo + 1, len(xs) - 1)
+    return xs[lo] + (xs[hi] - xs[lo]) * (pos - lo)
+
+
+def spread(xs):
+    return {"median": percentile(xs, 0.5), "p10": percentile(xs, 0.1), "p90": percentile(xs, 0.9), "samples": len(xs)}
+
+
+def read_traffic(cfg_id):
+    """HBM-side bytes per attention call from the committed counter summary of this configuration
+    (profiles/attn_ring_cfgN_hbm_traffic.txt: two rocprofv3 --pmc runs, FETCH_SIZE and WRITE_SIZE,
+    each scaled by the same counter's reading for a copy kernel of known size).  None when there is
+    no summary."""
+    path = os.path.join(ROOT, "profiles", f"attn_ring_cfg{cfg_id}_hbm_traffic.txt")
+    try:
+        text = open(path).read()
+    except OSError:
+        return None, None
+    m = re.search(r"traffic per attention call[^:]*:\s*([0-9]+)\s*bytes", text)
+    if not m:
+        return None, None
+    src = f"profiles/attn_ring_cfg{cfg_id}_hbm_traffic.txt"
+    rev = re.search(r"kernel sources at commit\s+([0-9a-f]{7,40})", text)
+    if rev:
+        src += f" (kernel sources at commit {rev.group(1)})"
+    return int(m.group(1)), src
+
+
+def cfg_namespace(c, layers):
+    from types import SimpleNamespace
+    return SimpleNamespace(tokens_per_frame=c["T"], local_window=c["slots"], global_window=c["slots"],
+                           global_attn_period=1, global_pinned_dilation=1, n_layers=layers,
+                           n_heads=c["H"], n_kv_heads=c["Hkv"], d_model=c["H"] * c["Dh"])
+
+
+def run_gpu(cfg_id, c, args, torch, ro, wea, ops):
+    """GPU legs of one configuration: the K-step schedule and the attention-only roofline timing."""
     B, H, Hkv, Dh, T, n, layers = c["B"], c["H"], c["Hkv"], c["Dh"], c["T"], c["slots"], c["layers"]
     L = n * T
     W = int(math.isqrt(T))
     dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
     dtype = torch.bfloat16
     K, Wm = args.steps, args.warmup
-    subs = c["frozen_subs"] + 1                      # attention calls per frame
-    frames_total = (Wm + K + subs - 1) // subs + n + 2
+    plan = schedule_plan(c, K, Wm)
+    subs = plan["subs"]
 
-    cache = wea.StaticKVCache(
-        __import__("types").SimpleNamespace(tokens_per_frame=T, local_window=n, global_window=n,
-                                            global_attn_period=1, global_pinned_dilation=1,
-                                            n_layers=layers, n_heads=H, n_kv_heads=Hkv, d_model=H * Dh),
-        B, dtype).to(dev)
+    cache = wea.StaticKVCache(cfg_namespace(c, layers), B, dtype).to(dev)
     for layer in cache.layers:
         layer.check_inputs = False                   # the eager sanity checks synchronise
-    cos, sin = ro.rope_table_1d(frames_total * T, Dh)
+    cos, sin = ro.rope_table_1d(plan["table_frames"] * T, Dh)
     rope = wea.RoPE(cos, sin, T // W, W).to(dev)
 
     # synthetic inputs, resident in HBM, in the merged-QKV layout the real module produces
     n_in = 4
     inputs = []
     for i in range(n_in):
-        q, k, v = ro.synth_qkv(args.config, i, 0, B, H, Hkv, T, Dh, dtype, outlier=c.get("outlier", False))
+        q, k, v = ro.synth_qkv(cfg_id, i, 0, B, H, Hkv, T, Dh, dtype, outlier=c.get("outlier", False))
         buf = torch.cat([q.transpose(1, 2).reshape(B, T, H * Dh), k.transpose(1, 2).reshape(B, T, Hkv * Dh),
                          v.transpose(1, 2).reshape(B, T, Hkv * Dh)], dim=-1).contiguous().to(dev)
         qq, kk, vv = buf.split((H * Dh, Hkv * Dh, Hkv * Dh), dim=-1)
@@ -127,10 +160,12 @@ def main():
     idx = torch.arange(T, dtype=torch.long)
     y_pos = (idx // W)[None].expand(B, T).contiguous().to(dev)
     x_pos = (idx % W)[None].expand(B, T).contiguous().to(dev)
-    t_pos_all = torch.arange(frames_total, dtype=torch.long)[:, None, None].expand(frames_total, B, T).contiguous().to(dev)
+    nf = plan["attn_frame"] + 1
+    t_pos_all = torch.arange(nf, dtype=torch.long)[:, None, None].expand(nf, B, T).contiguous().to(dev)
 
     n_splits = args.n_splits or ops.attn_auto_splits(B, H, Hkv, T, Dh, L)
-    ws = torch.empty(max(ops.attn_workspace_bytes(B, H, Hkv, T, Dh, L, args.n_splits, args.q_tile), 16), dtype=torch.uint8, device=dev)
+    ws = torch.empty(max(ops.attn_workspace_bytes(B, H, Hkv, T, Dh, L, args.n_splits, args.q_tile), 16),
+                     dtype=torch.uint8, device=dev)
     out = torch.empty((B, T, H, Dh), dtype=dtype, device=dev).transpose(1, 2)
 
     def one_step(step_idx):
@@ -165,22 +200,21 @@ def main():
         del src, dst
 
     # ---- fill the ring (untimed, not counted), then W warm-up steps ----
-    fill_steps = n * subs
-    for s in range(fill_steps):
-        one_step(s)
-    for s in range(fill_steps, fill_steps + Wm):
+    for s in range(plan["first"]):
         one_step(s)
     torch.cuda.synchronize()
-    first = fill_steps + Wm
+    first = plan["first"]
 
-    # ---- timed region: exactly K steps ----
+    # ---- timed region: exactly K steps per graph replay ----
     if args.eager:
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for s in range(first, first + K):
-            one_step(s)
-        torch.cuda.synchronize()
-        t1 = time.perf_counter()
+        def sample(reps):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                for s in range(first, first + K):
+                    one_step(s)
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) / reps
     else:
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
@@ -189,17 +223,26 @@ def main():
             for s in range(first, first + K):
                 one_step(s)
         torch.cuda.synchronize()                      # capture records, it does not execute
-        t0 = time.perf_counter()
-        graph.replay()
-        torch.cuda.synchronize()
-        t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / K
-    us_per_layer_step = ms_per_step * 1e3 / layers
-    log(f"[bench] {c['name']}: {ms_per_step * 1e3:.2f} us per step ({K} steps, n_splits={n_splits})")
+
+        def sample(reps):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                graph.replay()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) / reps
+    t_once = sample(1)                                # also a warm-up of the graph itself
+    t_once = sample(1)
+    reps = max(1, int(math.ceil(MIN_REGION_S / max(t_once, 1e-7))))
+    n_samples = 1 if args.eager else SAMPLES
+    per_step_us = [sample(reps) / K * 1e6 for _ in range(n_samples)]
+    st = spread(per_step_us)
+    log(f"[bench] {c['name']}: {st['median']:.2f} us per step (p10 {st['p10']:.2f}, p90 {st['p90']:.2f}; "
+        f"{K} steps x {reps} replays per sample, n_splits={n_splits})")
 
     # ---- attention-only timing at steady state for the roofline (HIP events on the launch stream) ----
     layer0 = cache.layers[0]
-    pos = {"t_pos": t_pos_all[(first + K) // subs + 1], "y_pos": y_pos, "x_pos": x_pos}
+    pos = {"t_pos": t_pos_all[plan["attn_frame"]], "y_pos": y_pos, "x_pos": x_pos}
     q_rot = ops.rope_kv_store(*inputs[0], pos, rope.cos, rope.sin, rope.height, rope.width,
                               layer0.kv, layer0.written, layer0.L, 1, True)
     iters = args.attn_iters
@@ -211,12 +254,15 @@ def main():
     for _ in range(5):
         attn_only()
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    attn_samples = []
     if args.eager:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(iters):
             attn_only()
         e1.record()
+        torch.cuda.synchronize()
+        attn_samples.append(e0.elapsed_time(e1) * 1e3 / iters)
     else:
         g2 = torch.cuda.CUDAGraph()
         side2 = torch.cuda.Stream()
@@ -227,11 +273,15 @@ def main():
         torch.cuda.synchronize()
         g2.replay()
         torch.cuda.synchronize()
-        e0.record()
-        g2.replay()
-        e1.record()
-    torch.cuda.synchronize()
-    attn_us = e0.elapsed_time(e1) * 1e3 / iters
+        for _ in range(SAMPLES):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            g2.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            attn_samples.append(e0.elapsed_time(e1) * 1e3 / iters)
+    ast = spread(attn_samples)
+    attn_us = ast["median"]
     n_vis = L                                        # steady state: n-1 ring slots + the tail
     flops, byts = algorithmic_work(c, n_vis)
     tflops = flops / (attn_us * 1e-6) / 1e12
@@ -242,92 +292,270 @@ def main():
     else:
         roof = {"bound": "mfma", "achieved": round(tflops, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(tflops / PEAK_BF16_TFLOPS, 4), "traffic": None}
-    if not (args.n_splits or args.q_tile or args.batch):
-        roof["traffic"] = MEASURED_TRAFFIC.get(args.config)
+    if not (args.n_splits or args.q_tile):
+        roof["traffic"], roof["traffic_source"] = read_traffic(cfg_id)
     roof.update({"kernel": "attn_ring_kernel" + (" + attn_combine_kernel" if n_splits > 1 else ""),
-                 "us_per_launch": round(attn_us, 3), "algorithmic_bytes": byts, "algorithmic_flops": flops,
-                 "n_splits": n_splits})
+                 "us_per_launch": round(attn_us, 3), "us_per_launch_p10": round(ast["p10"], 3),
+                 "us_per_launch_p90": round(ast["p90"], 3), "launches_per_sample": iters,
+                 "algorithmic_bytes": byts, "algorithmic_flops": flops, "n_splits": n_splits,
+                 "tflops": round(tflops, 2), "algorithmic_gbps": round(gbps, 1)})
     log(f"[bench] attention call: {attn_us:.2f} us -> {tflops:.1f} TFLOP/s, {gbps:.0f} GB/s algorithmic")
+    res = {"workload": c["name"], "us_per_step": round(st["median"], 3), "us_per_step_p10": round(st["p10"], 3),
+           "us_per_step_p90": round(st["p90"], 3), "samples": st["samples"], "replays_per_sample": reps,
+           "us_per_layer_step": round(st["median"] / layers, 3), "layers": layers, "calls_per_frame": subs,
+           "launch": "eager" if args.eager else "hip_graph", "n_splits": n_splits, "q_tile": args.q_tile or "auto",
+           "roofline": roof}
+    del cache, ws, out, inputs, t_pos_all
+    torch.cuda.empty_cache()
+    return res
 
-    # ---- CPU baseline: the oracle's restatement of the reference path on the host cores ----
-    cpu = None
-    if not args.no_cpu_baseline:
-        cfg1l = __import__("types").SimpleNamespace(tokens_per_frame=T, local_window=n, global_window=n,
-                                                    global_attn_period=1, global_pinned_dilation=1, n_layers=1,
-                                                    n_heads=H, n_kv_heads=Hkv, d_model=H * Dh)
-        oc = ro.OracleStaticKVCache(cfg1l, B, dtype)
+
+def run_cpu(cfg_id, c, args, torch, ro, threads=None, dtype=None, budget=None):
+    """CPU baseline: the oracle's restatement of the reference path (eager PyTorch on the host
+    cores), timed on a bounded sample of steady-state frame-steps of the same shape."""
+    B, H, Hkv, Dh, T, n, layers = c["B"], c["H"], c["Hkv"], c["Dh"], c["T"], c["slots"], c["layers"]
+    dtype = dtype or torch.bfloat16
+    W = int(math.isqrt(T))
+    plan = schedule_plan(c, args.steps, args.warmup)
+    cos, sin = ro.rope_table_1d(plan["table_frames"] * T, Dh)
+    old_threads = torch.get_num_threads()
+    if threads:
+        torch.set_num_threads(threads)
+    try:
+        oc = ro.OracleStaticKVCache(cfg_namespace(c, 1), B, dtype)   # one ring stands for every layer
         oc.set_frozen(False)
         oc.layers[0].kv.normal_()                    # steady state: every slot written
         oc.layers[0].written[:] = True
-        q, k, v = ro.synth_qkv(args.config, 0, 0, B, H, Hkv, T, Dh, dtype)
+        q, k, v = ro.synth_qkv(cfg_id, 0, 0, B, H, Hkv, T, Dh, dtype, outlier=c.get("outlier", False))
+        frames = plan["cpu_frames"]
+        assert max_table_row(max(frames), T) < cos.shape[0]
+        budget = budget if budget is not None else c["cpu_budget_s"]
+        ro.layer_step(oc, 0, q, k, v, ro.synth_pos_ids(frames[0], B, T, W), cos, sin, T // W, W)   # untimed warm-up
         done, spent = 0, 0.0
-        budget = 12.0 if c["B"] * c["H"] * c["T"] <= 16 * 256 else 20.0
-        ro.layer_step(oc, 0, q, k, v, ro.synth_pos_ids(n, B, T, W), cos, sin, T // W, W)   # untimed warm-up
-        while spent < budget and done < 1000:    # about 12 s of host work (20 s for the large shapes)
-            pos_c = ro.synth_pos_ids(n + 1 + done, B, T, W)
+        while (spent < budget and done < 1000) or done < 2:
+            pos_c = ro.synth_pos_ids(frames[done % len(frames)], B, T, W)
             t0c = time.perf_counter()
             ro.layer_step(oc, 0, q, k, v, pos_c, cos, sin, T // W, W)
             spent += time.perf_counter() - t0c
             done += 1
-        cpu = {"value": round(spent / done * 1e6, 1), "unit": "us per frame-step (one layer)",
-               "cores": torch.get_num_threads(), "kind": "port",
-               "sample": f"{done} steady-state frame-steps of the same shape through oracle/ring_oracle.layer_step "
-                         f"(eager PyTorch CPU, bf16 inputs, fp32 scores), host cpu_count={os.cpu_count()}"}
-        log(f"[bench] cpu baseline: {cpu['value']:.0f} us per frame-step on {cpu['cores']} threads")
+        per_layer_us = spent / done * 1e6
+        return {"value": round(per_layer_us * layers, 1), "unit": "us per frame-step"
+                + (f" ({layers} layers = {layers} x the measured one-layer step)" if layers > 1 else " (one layer)"),
+                "cores": torch.get_num_threads(), "kind": "port",
+                "sample": f"{done} steady-state one-layer frame-steps of the same shape through "
+                          f"oracle/ring_oracle.layer_step (eager PyTorch CPU, {str(dtype).replace('torch.', '')} inputs, "
+                          f"fp32 scores), {spent:.1f} s of host work, host cpu_count={os.cpu_count()}"}
+    finally:
+        torch.set_num_threads(old_threads)
 
-    peaks = None
-    if args.peaks:
-        # achievable rates on this box next to the published ones the roofline is priced against
-        a = torch.randn(8192, 8192, device=dev, dtype=dtype)
-        b2 = torch.randn(8192, 8192, device=dev, dtype=dtype)
-        src = torch.empty(1 << 28, dtype=torch.int32, device=dev)          # 1 GiB
-        dst = torch.empty_like(src)
 
-        def timed(fn, n):
-            for _ in range(3):
-                fn()
+def run_module(args, torch, ro, wea):
+    """The attention module around the path at cfg1 shapes (d_model 2048, merged QKV projection,
+    value residual and head gate, output projection), 20 layers' worth in one HIP graph: with the
+    element-wise neighbours as torch operations and with them inside the kernels."""
+    from types import SimpleNamespace
+    dev = torch.device("cuda:0")
+    T, H, Dh, n = 256, 16, 128, 16
+    cfg = SimpleNamespace(d_model=H * Dh, n_heads=H, n_kv_heads=H, value_residual=True, gated_attn=True,
+                          tokens_per_frame=T, local_window=n, global_window=n, global_attn_period=1,
+                          global_pinned_dilation=1, n_layers=1)
+    cos, sin = ro.rope_table_1d(64 * T, Dh)
+    rope = wea.RoPE(cos, sin, 16, 16).to(dev)
+    res = {}
+    for fuse in (False, True):
+        torch.manual_seed(0)
+        mod = wea.RingAttn(cfg, 0, rope, merged_qkv=True, fuse_elementwise=fuse).to(dev, torch.bfloat16)
+        cache = wea.StaticKVCache(cfg, 1, torch.bfloat16).to(dev)
+        cache.set_frozen(False)
+        for layer in cache.layers:
+            layer.check_inputs = False
+        x = torch.randn(1, T, H * Dh, device=dev, dtype=torch.bfloat16)
+        v1 = torch.randn(1, H, T, Dh, device=dev, dtype=torch.bfloat16)
+        poss = [{k: v.to(dev) for k, v in ro.synth_pos_ids(t, 1, T, 16).items()} for t in range(40)]
+        with torch.no_grad():
+            for t in range(20):
+                mod(x, poss[t], v1, cache)
             torch.cuda.synchronize()
-            s0, s1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            s0.record()
-            for _ in range(n):
-                fn()
-            s1.record()
+            g = torch.cuda.CUDAGraph()
+            s = torch.cuda.Stream()
+            s.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.graph(g, stream=s):
+                for t in range(20, 40):
+                    mod(x, poss[t], v1, cache)
             torch.cuda.synchronize()
-            return s0.elapsed_time(s1) * 1e-3 / n
+            g.replay()
+            torch.cuda.synchronize()
+            xs = []
+            for _ in range(SAMPLES):
+                t0 = time.perf_counter()
+                for _ in range(10):
+                    g.replay()
+                torch.cuda.synchronize()
+                xs.append((time.perf_counter() - t0) / 200 * 1e6)
+        res["fused_elementwise" if fuse else "torch_elementwise"] = round(percentile(xs, 0.5), 2)
+        del mod, cache, g
+    res["what"] = ("us per RingAttn.forward at cfg1 shapes (d_model 2048, merged qkv_proj, value residual, head gate, "
+                   "out_proj included), 20 calls per HIP graph")
+    return res
 
-        t_mm = timed(lambda: torch.matmul(a, b2), 20)
-        t_cp = timed(lambda: torch.add(src, 0, out=dst), 20)
-        peaks = {"bf16_gemm_8192_tflops": round(2 * 8192 ** 3 / t_mm / 1e12, 1),
-                 "copy_1gib_read_plus_write_gbps": round(2 * src.numel() * 4 / t_cp / 1e9, 1)}
-        log(f"[bench] measured on this box: {peaks}")
-        del a, b2, src, dst
 
+def run_peaks(torch):
+    """What this box reaches on library code, next to the published peaks the roofline is priced
+    against: a bf16 GEMM through hipBLASLt and a streaming copy."""
+    dev = torch.device("cuda:0")
+    a = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
+    b2 = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
+    src = torch.empty(1 << 28, dtype=torch.int32, device=dev)          # 1 GiB
+    dst = torch.empty_like(src)
+
+    def timed(fn, n):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        s0, s1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s0.record()
+        for _ in range(n):
+            fn()
+        s1.record()
+        torch.cuda.synchronize()
+        return s0.elapsed_time(s1) * 1e-3 / n
+
+    t_mm = timed(lambda: torch.matmul(a, b2), 20)
+    t_cp = timed(lambda: torch.add(src, 0, out=dst), 20)
+    peaks = {"bf16_gemm_8192_tflops": round(2 * 8192 ** 3 / t_mm / 1e12, 1),
+             "copy_1gib_read_plus_write_gbps": round(2 * src.numel() * 4 / t_cp / 1e9, 1)}
+    del a, b2, src, dst
+    torch.cuda.empty_cache()
+    return peaks
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--config", type=int, default=0, choices=[0] + sorted(CONFIGS),
+                    help="0 (default): configurations 1-4 in one run, configuration 1 at the top level; N: only N")
+    ap.add_argument("--n-splits", type=int, default=0, help="context splits (0 = library's choice)")
+    ap.add_argument("--q-tile", type=int, default=0, help="queries per workgroup (0 = library's choice)")
+    ap.add_argument("--eager", action="store_true", help="launch from Python per call instead of a HIP graph")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-module", action="store_true", help="skip the module-level timing")
+    ap.add_argument("--no-peaks", action="store_true", help="skip the measured GEMM / copy rates of this box")
+    ap.add_argument("--two-calls", action="store_true",
+                    help="we_rope_kv_store + we_attn_ring_fwd instead of the one-call we_rope_kv_attn_fwd")
+    ap.add_argument("--attn-iters", type=int, default=200, help="attention-only launches for the roofline timing")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
+                    help="also launch 20 plain copy kernels (read MiB, write MiB each) so a counter run holds "
+                         "a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
+    args = ap.parse_args()
+
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures the single-GPU hot path only: this build has no multi-GPU path "
+              "(heads and batch streams would shard with no communication); run with --gpus 1.",
+              file=sys.stderr)
+        sys.exit(2)
+    if args.steps < 1 or args.warmup < 0:
+        print("--steps must be >= 1 and --warmup >= 0", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from oracle import ring_oracle as ro           # inputs + the cpu_baseline leg only
+    import world_engine_amd as wea
+    from world_engine_amd import ops
+
+    torch.cuda.set_device(0)
+    single = args.config != 0
+    cfg_ids = [args.config] if single else sorted(CONFIGS)
+    head = args.config if single else HEADLINE
+    profiling = single or args.eager or args.calibrate_copy
+
+    # ---- GPU legs first: nothing on the host can lose them afterwards ----
+    per_cfg = {}
+    extras = {}
+    failures = []
+    for cid in cfg_ids:
+        try:
+            per_cfg[cid] = run_gpu(cid, CONFIGS[cid], args, torch, ro, wea, ops)
+        except Exception as e:                      # noqa: BLE001 - reported in the line
+            traceback.print_exc()
+            failures.append(f"gpu cfg{cid}: {e!r}")
+    if not profiling and not args.no_peaks:
+        try:
+            extras["measured_peaks"] = run_peaks(torch)
+            log(f"[bench] measured on this box: {extras['measured_peaks']}")
+        except Exception as e:                      # noqa: BLE001
+            failures.append(f"measured_peaks: {e!r}")
+    if not profiling and not args.no_module:
+        try:
+            extras["module"] = run_module(args, torch, ro, wea)
+            log(f"[bench] module: {extras['module']}")
+        except Exception as e:                      # noqa: BLE001
+            failures.append(f"module: {e!r}")
+
+    h = per_cfg.get(head)
     result = {
         "metric": "attn_us_per_frame_step",
-        "value": round(ms_per_step * 1e3, 3),
+        "value": h["us_per_step"] if h else None,
         "unit": "us",
         "n_gpus": 1,
-        "steps": K,
-        "warmup": Wm,
-        "ms_per_step": round(ms_per_step, 6),
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(h["us_per_step"] * 1e-3, 6) if h else None,
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": c["name"], "launch": "eager" if args.eager else "hip_graph",
-                   "calls_per_step": f"{layers} x " + ("(we_rope_kv_store + we_attn_ring_fwd)" if args.two_calls
-                                                       else "we_rope_kv_attn_fwd (store kernel + attention kernels)"),
-                   "n_splits": n_splits, "q_tile": args.q_tile or "auto"},
-        "us_per_layer_step": round(us_per_layer_step, 3),
-        "attn_tflops": round(tflops, 2),
-        "attn_algorithmic_gbps": round(gbps, 1),
-        "roofline": roof,
-        "cpu_baseline": cpu,
+        "config": {"workload": CONFIGS[head]["name"],
+                   "why": "the configuration the metric is quoted on (second entry of the benchmark list); the two "
+                          "stated targets are on cfg3 (MFMA) and cfg4 (HBM), whose figures are under configs",
+                   "calls_per_step": f"{CONFIGS[head]['layers']} x "
+                                     + ("(we_rope_kv_store + we_attn_ring_fwd)" if args.two_calls
+                                        else "we_rope_kv_attn_fwd (store kernel + attention kernels)")},
+        "roofline": None,
+        "cpu_baseline": None,
+        "configs": {f"cfg{cid}": per_cfg[cid] for cid in cfg_ids if cid in per_cfg},
     }
-    if peaks is not None:
-        result["measured_peaks"] = peaks
+    if h:
+        result["config"].update({
+            "launch": h["launch"], "n_splits": h["n_splits"], "q_tile": h["q_tile"],
+            "timing": f"median of {h['samples']} samples, each {h['replays_per_sample']} back-to-back replays of a "
+                      f"{args.steps}-step HIP graph between device synchronisations"})
+        result.update({"p10": h["us_per_step_p10"], "p90": h["us_per_step_p90"],
+                       "us_per_layer_step": h["us_per_layer_step"], "attn_tflops": h["roofline"]["tflops"],
+                       "attn_algorithmic_gbps": h["roofline"]["algorithmic_gbps"], "roofline": h["roofline"]})
+    result.update(extras)
+
+    # ---- CPU baselines: the oracle's restatement of the reference path on the host cores ----
+    if not (args.no_cpu_baseline or args.eager or args.calibrate_copy):
+        for cid in cfg_ids:
+            if cid not in per_cfg:
+                continue
+            try:
+                cpu = run_cpu(cid, CONFIGS[cid], args, torch, ro)
+                per_cfg[cid]["cpu_baseline"] = cpu
+                log(f"[bench] cpu baseline cfg{cid}: {cpu['value']:.0f} us per frame-step on {cpu['cores']} threads")
+            except Exception as e:                  # noqa: BLE001
+                traceback.print_exc()
+                per_cfg[cid]["cpu_baseline"] = None
+                failures.append(f"cpu_baseline cfg{cid}: {e!r}")
+        if h:
+            result["cpu_baseline"] = h.get("cpu_baseline")
+        try:
+            c = CONFIGS[head]
+            one = run_cpu(head, c, args, torch, ro, threads=1, budget=3.0)
+            f32 = run_cpu(head, c, args, torch, ro, dtype=torch.float32, budget=3.0)
+            result["cpu_baseline_variants"] = {"one_thread": one, "fp32_inputs": f32}
+            log(f"[bench] cpu baseline cfg{head}: {one['value']:.0f} us on 1 thread, {f32['value']:.0f} us with fp32 inputs")
+        except Exception as e:                      # noqa: BLE001
+            traceback.print_exc()
+            failures.append(f"cpu_baseline variants: {e!r}")
+    if failures:
+        result["failures"] = failures
     print(json.dumps(result), flush=True)
+    if failures:
+        sys.exit(1)
 
 
 if __name__ == "__main__":

@@ -32,7 +32,7 @@ extern "C" {
 /* element types of q/k/v, the cache buffer and the attention output */
 #define WE_DTYPE_BF16 0
 #define WE_DTYPE_F16 1
-#define WE_DTYPE_F32 2 /* we_rope_kv_store only */
+#define WE_DTYPE_F32 2 /* fp32 caches: the store rotates in fp32, the attention takes a plain one-pass kernel */
 
 #define WE_OK 0
 #define WE_ERR_NULL_POINTER (-1)
@@ -65,8 +65,11 @@ const char* we_error_string(int code);
  *            given, q is copied), which is the behaviour of StaticKVCache.upsert on an already
  *            rotated k.
  *   t_pos, y_pos, x_pos   int64 [B, T], row stride pos_stride_b.  Table row of token (b, i) is
- *            t_pos*grid_h*grid_w + y_pos*grid_w + x_pos (src/model/attn.py:27), clamped into
- *            [0, table_rows).  y_pos/x_pos may be NULL when the tables are NULL.
+ *            t_pos*grid_h*grid_w + y_pos*grid_w + x_pos (src/model/attn.py:27).  The kernel clamps
+ *            it into [0, table_rows) for memory safety only: a row outside the table is a caller
+ *            error (the reference's index_select raises there, src/model/attn.py:25-30), which the
+ *            Python wrapper checks in eager mode; the C entry point cannot without reading device
+ *            memory.  y_pos/x_pos may be NULL when the tables are NULL.
  *            t_pos[0] is the frame index that selects the ring slot.
  *   kv       [2, B, Hkv, L + T, Dh] contiguous cache buffer (plane 0 = K, 1 = V).
  *   written  [L + T] bytes (torch.bool).

@@ -282,3 +282,23 @@ int main(void) {
     assert int(rc_null) == -1                                    # WE_ERR_NULL_POINTER
     assert int(ws) == 4 * 16 * 256 * (128 * 2 + 8)
     assert "workspace" in msg
+
+
+def test_rope_position_ids_are_bounds_checked_in_eager_mode():
+    """The reference asserts y < height, x < width and its index_select raises on a table row past
+    the end (src/model/attn.py:25-30); the kernels only clamp, so the host check must raise."""
+    from oracle import ring_oracle as ro
+    rope = wea.RoPE.one_dimensional(4 * 16, 32, 4, 4)            # rows for frames 0..3 of a 4x4 grid
+    rope.check_pos_ids(ro.synth_pos_ids(3, 1, 16, 4))            # last frame the table holds
+    with pytest.raises(IndexError, match="index out of range"):
+        rope.check_pos_ids(ro.synth_pos_ids(4, 1, 16, 4))        # one frame past the table
+    with pytest.raises(AssertionError, match="pos_ids out of bounds"):
+        rope.check_pos_ids(ro.synth_pos_ids(0, 1, 16, 2))        # y runs to 7 on a grid of height 4
+    neg = ro.synth_pos_ids(0, 1, 16, 4)
+    neg["t_pos"] = neg["t_pos"] - 1
+    with pytest.raises(IndexError):
+        rope.check_pos_ids(neg)
+    # the oracle raises on the same inputs (index_select), so both sides fail alike
+    cos, sin = ro.rope_table_1d(4 * 16, 32)
+    with pytest.raises((IndexError, RuntimeError)):
+        ro.rope_angles(ro.synth_pos_ids(4, 1, 16, 4), cos, sin, 4, 4)

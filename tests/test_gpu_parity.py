@@ -235,6 +235,31 @@ def test_attention_cfg2_outlier_channel_three_layers(gpu_device):
             assert_attn_close(out, ro.attention_fp32(q_o, k_all, v_all, mask), f"cfg2 t={t} layer={layer}")
 
 
+def test_attention_cfg2_full_depth_24_layers(gpu_device):
+    """Benchmark configuration 2 at full depth: 24 layers, each with its own 16-slot ring (856 MB in
+    all), one K channel x8, 19 frames (the ring wraps after 16).  Cache buffers and `written` of
+    all 24 layers are compared bit for bit after every frame; the attention of four layers per
+    frame (rotating, so every layer is covered) against the fp32 oracle."""
+    L_ = 24
+    p = Pair(gpu_device, torch.bfloat16, B=1, H=16, Hkv=16, T=256, Dh=128, n_slots=16, n_layers=L_, cfg_id=2)
+    p.set_frozen(False)
+    worst = (0.0, 0.0)
+    for t in range(19):
+        _say(f"cfg2 full depth: frame {t}")
+        pos = ro.synth_pos_ids(t, 1, 256, 16)
+        checked = {(4 * t + i) % L_ for i in range(4)}
+        for layer in range(L_):
+            q, k, v = ro.synth_qkv(2, t, layer, 1, 16, 16, 256, 128, torch.bfloat16, outlier=True)
+            (q_o, k_all, v_all, mask), (q_h, ring) = p.store(q, k, v, pos, layer=layer)
+            out = p.attend(q_h, ring)
+            if layer in checked:
+                mx, mean = assert_attn_close(out, ro.attention_fp32(q_o, k_all, v_all, mask), f"cfg2 t={t} layer={layer}")
+                worst = (max(worst[0], mx), max(worst[1], mean))
+        for layer in range(L_):
+            p.assert_state_equal(layer=layer, what=f"t={t} layer={layer}")
+    _say(f"cfg2 full depth: worst max-abs {worst[0]:.2e} mean-abs {worst[1]:.2e}")
+
+
 def test_attention_cfg4_frozen_substeps_schedule(gpu_device):
     """Benchmark configuration 4: 32 slots, 4 frozen substeps re-attending the same ring + 1 persisting
     call per frame.  State is compared after every call; outputs on the first frames and around
@@ -399,6 +424,23 @@ def test_bad_inputs_raise(gpu_device):
     bad["t_pos"].fill_(-1)
     with pytest.raises(RuntimeError, match="non-negative"):
         p.hip.upsert(k.to(dev), v.to(dev), bad, 0)
+    # a RoPE table that is too short for the frame index raises instead of clamping
+    # (src/model/attn.py:25-30: index_select on the flat position)
+    short = wea.RoPE(*ro.rope_table_1d(2 * 64, 64), p.Hgrid, p.W).to(dev)
+    good = to_dev(p.inputs(1)[3], dev)
+    late = to_dev(p.inputs(2)[3], dev)
+    p.hip.rope_upsert(q.to(dev), k.to(dev), v.to(dev), good, short, 0)
+    before = p.hip.layers[0].kv.clone()
+    with pytest.raises(IndexError, match="index out of range"):
+        p.hip.rope_upsert(q.to(dev), k.to(dev), v.to(dev), late, short, 0)
+    with pytest.raises(IndexError, match="index out of range"):
+        p.hip.rope_upsert_attend(q.to(dev), k.to(dev), v.to(dev), late, short, 0)
+    with pytest.raises(IndexError, match="index out of range"):
+        short(q.to(dev), late)
+    assert torch.equal(p.hip.layers[0].kv, before), "a refused call must not touch the cache"
+    narrow = wea.RoPE(*ro.rope_table_1d(64 * 64, 64), p.Hgrid // 2, p.W).to(dev)
+    with pytest.raises(AssertionError, match="pos_ids out of bounds"):
+        p.hip.rope_upsert(q.to(dev), k.to(dev), v.to(dev), good, narrow, 0)
     # unsupported head dim for the attention kernel
     layer = wea.LayerKVCache(1, 1, 64, 32, torch.bfloat16, 64).to(dev)
     with pytest.raises(RuntimeError, match="not covered"):

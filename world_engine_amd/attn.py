@@ -4,9 +4,10 @@
 ``src/patch_model.py:92-141``): same parameters and state-dict keys, same call signature, same
 order of operations.  The part between the q/k/v projection and the output projection - RoPE,
 cache update, masked attention - runs as two HIP kernel launches (three with context splits)
-instead of the reference's eager/compiled op sequence.  Projections, the weightless RMS norm,
-the value-residual lerp and the head gate stay ordinary torch ops; they are the neighbours of
-the path, not the path.
+instead of the reference's eager/compiled op sequence.  Projections stay ordinary torch ops.  The
+weightless RMS norm, the value-residual lerp and the head gate are torch ops by default and move
+into the two kernels with ``fuse_elementwise=True`` (results then agree to 1 ulp instead of bit
+for bit).
 """
 from __future__ import annotations
 
@@ -80,7 +81,25 @@ class RoPE(nn.Module):
         ], dim=-1).reshape(n_frames * height * width, d_head // 2)
         return cls(table.cos(), table.sin(), height, width)
 
+    def check_pos_ids(self, pos_ids: Mapping[str, Tensor]) -> None:
+        """Eager-mode bounds check of the position ids, as the reference's ``get_angles`` has it
+        (``src/model/attn.py:25-30``): ``y < height`` and ``x < width`` are asserted, and a table
+        row past the end raises like its ``index_select``.  The kernels clamp the row for memory
+        safety only, so without this check a table that is too short would rotate by wrong angles
+        silently.  Synchronises; skipped under ``torch.compile`` and stream capture."""
+        t, y, x = pos_ids["t_pos"], pos_ids["y_pos"], pos_ids["x_pos"]
+        if torch.compiler.is_compiling() or (t.is_cuda and torch.cuda.is_current_stream_capturing()):
+            return
+        flat = t * (self.height * self.width) + y * self.width + x
+        y_max, x_max, f_min, f_max = (int(v) for v in torch.stack([y.max(), x.max(), flat.min(), flat.max()]).tolist())
+        if not (y_max < self.height and x_max < self.width):
+            raise AssertionError(f"pos_ids out of bounds, {y_max}, {x_max}")
+        if f_min < 0 or f_max >= self.cos.shape[0]:
+            raise IndexError(f"index out of range in self: RoPE table has {self.cos.shape[0]} rows, position ids "
+                             f"select rows {f_min}..{f_max}")
+
     def forward(self, x: Tensor, pos_ids: Mapping[str, Tensor]) -> Tensor:
+        self.check_pos_ids(pos_ids)
         return ops.rope_apply(x, pos_ids, self.cos, self.sin, self.height, self.width)
 
 

@@ -77,7 +77,7 @@ class LayerKVCache(nn.Module):
         self.written[self.L:].fill_(True)
 
     # -- input checks of the reference's eager path (src/model/kv_cache.py:112-124) ------------
-    def _check(self, k: Tensor, pos_ids: Mapping[str, Tensor]) -> None:
+    def _check(self, k: Tensor, pos_ids: Mapping[str, Tensor], rope=None) -> None:
         t_pos = pos_ids["t_pos"]
         ops._need_device(k, self.kv, t_pos)
         if k.size(2) != self.tpf:
@@ -89,6 +89,8 @@ class LayerKVCache(nn.Module):
                 raise RuntimeError("t_pos must be non-negative during inference")
             if not bool((t_pos == t_pos[:, :1]).all().item()):
                 raise RuntimeError("t_pos must be constant within frame")
+            if rope is not None:   # the bounds check of the reference's RoPE (src/model/attn.py:25-30)
+                rope.check_pos_ids(pos_ids)
 
     def _mask(self, pos_ids: Mapping[str, Tensor]) -> RingMask:
         return RingMask(self.kv, self.written, pos_ids["t_pos"], self.L, self.tpf, self.pinned_dilation)
@@ -108,7 +110,7 @@ class LayerKVCache(nn.Module):
                     is_frozen: bool):
         """Fused path used by the attention module: rotate q and k with ``rope``'s tables, store
         k/v, return ``(RoPE(q), k_all, v_all, mask)`` from a single kernel launch."""
-        self._check(k, pos_ids)
+        self._check(k, pos_ids, rope)
         q_rot = ops.rope_kv_store(q, k, v, pos_ids, rope.cos, rope.sin, rope.height, rope.width,
                                   self.kv, self.written, self.L, self.pinned_dilation, is_frozen)
         return q_rot, self.kv[0], self.kv[1], self._mask(pos_ids)
@@ -126,7 +128,7 @@ class LayerKVCache(nn.Module):
                 q, k, v, pos_ids["t_pos"], pos_ids["y_pos"], pos_ids["x_pos"], rope.cos, rope.sin, rope.height,
                 rope.width, self.kv, self.written, self.L, self.pinned_dilation, bool(is_frozen), s,
                 float(qk_norm_eps), v1, v_lamb, gate)
-        self._check(k, pos_ids)
+        self._check(k, pos_ids, rope)
         return ops.rope_kv_attn(q, k, v, pos_ids, rope.cos, rope.sin, rope.height, rope.width, self.kv,
                                 self.written, self.L, self.pinned_dilation, is_frozen, scale,
                                 qk_norm_eps=qk_norm_eps, v1=v1, v_lamb=v_lamb, gate=gate)[0]
