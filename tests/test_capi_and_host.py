@@ -65,15 +65,15 @@ def test_validation_codes_without_gpu():
 def test_workspace_and_split_planning():
     lib = _capi.lib()
     assert lib.we_attn_workspace_bytes(1, 16, 16, 256, 128, 4096, 1, 0) == 0
-    assert lib.we_attn_workspace_bytes(1, 16, 16, 256, 128, 4096, 4, 0) == 4 * 16 * 256 * (128 * 2 + 8)
+    assert lib.we_attn_workspace_bytes(1, 16, 16, 256, 128, 4096, 4, 0) == 4 * 16 * 256 * (128 * 2 + 16)
     # 256-token frames: every unit is split so that all 256 CUs have work
     s = lib.we_attn_auto_splits(1, 16, 16, 256, 128, 4096)
     assert s == 8
-    assert lib.we_attn_workspace_bytes(1, 16, 16, 256, 128, 4096, 0, 0) == s * 16 * 256 * (128 * 2 + 8)
+    assert lib.we_attn_workspace_bytes(1, 16, 16, 256, 128, 4096, 0, 0) == s * 16 * 256 * (128 * 2 + 16)
     # 1024-token frames with 96 heads: 384 workgroups of 256 queries = 1.5 rounds of 256 CUs, so only
     # the last 32 of the 96 units (128 workgroups) are split in two
     assert lib.we_attn_auto_splits(4, 24, 24, 1024, 128, 8192) == 2
-    assert lib.we_attn_workspace_bytes(4, 24, 24, 1024, 128, 8192, 0, 0) == 2 * 32 * 1024 * (128 * 2 + 8)
+    assert lib.we_attn_workspace_bytes(4, 24, 24, 1024, 128, 8192, 0, 0) == 2 * 32 * 1024 * (128 * 2 + 16)
     # whole rounds: nothing to split
     assert lib.we_attn_auto_splits(4, 32, 32, 1024, 128, 8192) == 1
     assert lib.we_attn_workspace_bytes(4, 32, 32, 1024, 128, 8192, 0, 0) == 0
@@ -280,7 +280,7 @@ int main(void) {
     lib = _capi.lib()
     assert int(version) == lib.we_version()
     assert int(rc_null) == -1                                    # WE_ERR_NULL_POINTER
-    assert int(ws) == 4 * 16 * 256 * (128 * 2 + 8)
+    assert int(ws) == 4 * 16 * 256 * (128 * 2 + 16)
     assert "workspace" in msg
 
 

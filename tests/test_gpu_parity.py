@@ -185,6 +185,31 @@ def test_attention_frame_lengths_off_the_tile_grid(gpu_device, T, Dh, kw):
     _run_and_check(p, 8, frozen_subs=1, **kw)
 
 
+@pytest.mark.parametrize("T,n_slots,kw", [(8, 3, {}), (24, 2, {"n_splits": 2}), (96, 3, {"n_splits": 4}),
+                                          (96, 3, {"n_splits": 1, "q_tile": 128}), (64, 3, {"n_splits": 2}),
+                                          (256, 4, {})])
+def test_attention_all_logits_far_below_zero(gpu_device, T, n_slots, kw):
+    """Every logit is near -290 in the log2 domain (one channel of q and k carries +48 / -48): a
+    softmax only sees differences, so the result is an ordinary one, but any reference exponent
+    that is not taken from the data (a wavefront that starts on an empty 32-key block of a short
+    tile, a split without keys) would make every probability underflow to zero.  With 96-token
+    frames and 4 splits two of the splits start on the short second tile of a slot."""
+    p = Pair(gpu_device, torch.bfloat16, B=1, H=2, Hkv=2, T=T, Dh=128, n_slots=n_slots, cfg_id=27)
+    p.set_frozen(False)
+    for t in range(n_slots + 2):
+        q, k, v, pos = p.inputs(t)
+        q[..., 126] = 48.0
+        k[..., 126] = -48.0
+        (q_o, k_all, v_all, mask), (q_h, ring) = p.store(q, k, v, pos)
+        out = p.attend(q_h, ring, **kw)
+        p.assert_state_equal(what=f"t={t}")
+        ref = ro.attention_fp32(q_o, k_all, v_all, mask)
+        s = (q_o.float() @ k_all.float().transpose(-1, -2))[..., mask] * (128 ** -0.5) * 1.4427
+        assert s.max().item() < -200.0
+        assert ref.abs().max().item() > 0.1
+        assert_attn_close(out, ref, f"T={T} t={t} {kw}")
+
+
 def test_attention_fp32_ragged_frame(gpu_device):
     p = Pair(gpu_device, torch.float32, B=1, H=2, Hkv=2, T=72, Dh=64, n_slots=3, cfg_id=52)
     for t in range(7):
@@ -211,7 +236,7 @@ def test_attention_partial_round_tail_split(gpu_device):
     """320 workgroups = one full round of 256 CUs plus a quarter round: the library splits the
     context of the last 32 heads only (mixed direct-output and workspace rows in one call)."""
     assert ops.attn_auto_splits(1, 160, 160, 256, 64, 512) == 2
-    assert ops.attn_workspace_bytes(1, 160, 160, 256, 64, 512) == 2 * 32 * 256 * (64 * 2 + 8)
+    assert ops.attn_workspace_bytes(1, 160, 160, 256, 64, 512) == 2 * 32 * 256 * (64 * 2 + 16)
     p = Pair(gpu_device, torch.bfloat16, B=1, H=160, Hkv=160, T=256, Dh=64, n_slots=2, cfg_id=27)
     _run_and_check(p, 4)
 

@@ -1,35 +1,58 @@
-"""Build ``libwe_attn.so`` (HIP, gfx950) in-tree: ``python -m world_engine_amd.build``."""
+"""Build ``libwe_attn.so`` (HIP, gfx950) in-tree: ``python -m world_engine_amd.build``.
+
+Every source is compiled to its own object, in parallel (the main attention kernel once per
+element type / head dim family), and the objects are linked into the shared library."""
 from __future__ import annotations
 
 import os
 import subprocess
 import sys
+from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
-SOURCES = ["rope_kv_store.hip", "attn_ring.hip", "attn_ring_f32.hip", "attn_combine.hip", "capi.hip"]
+OBJ_DIR = os.path.join(HERE, "_obj")
+# (source, extra defines, object name)
+UNITS = [("rope_kv_store.hip", [], "rope_kv_store.o"),
+         ("attn_ring.hip", ["-DWE_RING_PART=0"], "attn_ring_bf16_128.o"),
+         ("attn_ring.hip", ["-DWE_RING_PART=1"], "attn_ring_bf16_64.o"),
+         ("attn_ring.hip", ["-DWE_RING_PART=2"], "attn_ring_f16_128.o"),
+         ("attn_ring.hip", ["-DWE_RING_PART=3"], "attn_ring_f16_64.o"),
+         ("attn_ring_f32.hip", [], "attn_ring_f32.o"),
+         ("attn_combine.hip", [], "attn_combine.o"),
+         ("capi.hip", [], "capi.o")]
+SOURCES = sorted({u[0] for u in UNITS})
 OUT = os.path.join(HERE, "libwe_attn.so")
 
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # keep fp32 arithmetic scalar: packed fp32 instructions are avoided on purpose
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
 
 
-def build(verbose: bool = False) -> str:
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc, *HIPCC_FLAGS, *[os.path.join(CSRC, s) for s in SOURCES], "-o", OUT]
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
-    noise = "packed-fp32-ops"
-    err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
+    noise = ("packed-fp32-ops", "Reserved registers on the clobber list", "warnings generated", "warning generated")
+    lines = res.stderr.splitlines()
+    err = "\n".join(l for l in lines if not any(n in l for n in noise))
     if res.returncode != 0:
-        raise RuntimeError(f"hipcc failed ({res.returncode}):\n{err}")
-    if verbose and err.strip():
-        print(err, file=sys.stderr)
+        raise RuntimeError(f"hipcc failed ({res.returncode}): {' '.join(cmd)}\n{err}")
+    return err
+
+
+def build(verbose: bool = False, jobs: int = 8) -> str:
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    cmds = [[hipcc, *HIPCC_FLAGS, *defs, "-c", os.path.join(CSRC, src), "-o", os.path.join(OBJ_DIR, obj)]
+            for src, defs, obj in UNITS]
+    with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(cmds)))) as pool:
+        list(pool.map(lambda c: _run(c, verbose), cmds))
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *[os.path.join(OBJ_DIR, u[2]) for u in UNITS], "-o", OUT],
+         verbose)
     return OUT
 
 

@@ -1,6 +1,6 @@
 // Second pass of split-context attention over the KV ring buffer (gfx950): merges the per-split
 // partial results the main kernel (attn_ring.hip) leaves in the workspace.
-// HBM-bound: reads n_splits * (Dh * 2 + 8) bytes and writes Dh * 2 bytes per query row that was
+// HBM-bound: reads n_splits * (Dh * 2 + 16) bytes and writes Dh * 2 bytes per query row that was
 // split.
 #include "attn_mma.h"
 #include "we_kernels.h"
@@ -9,8 +9,9 @@
 namespace we {
 
 // Second pass of the split-context path.  Every split left, per query row, its normalised
-// output O_s (element type), its reference m_s (log2 domain) and its sum l_s; the result is
-// sum_s w_s O_s / sum_s w_s with w_s = 2^(m_s - max m) * l_s.  One thread per (row, 8 columns);
+// output as fp16 values in [-1, 1] times a row scale r_s, its reference m_s (log2 domain) and its
+// sum l_s; the result is sum_s w_s r_s O_s / sum_s w_s with w_s = 2^(m_s - max m) * l_s.  One
+// thread per (row, 8 columns);
 // grid = (256-thread slices of one head's T * DH/8 items, split (batch, head) pairs), so that the
 // start-up code has one 32-bit division in it (the kernel is short enough for that to show).
 template <typename M, int DH>
@@ -28,27 +29,28 @@ __global__ void __launch_bounds__(256) attn_combine_kernel(AttnParams p) {
 #pragma unroll
   for (int j = 0; j < 8; ++j) acc[j] = 0.f;
   for (int s0 = 0; s0 < p.n_splits; s0 += 8) {
-    float2 ml[8];
-    frag_t ov[8];
+    f32x4_t ml[8];   // (m, l, row scale, -)
+    f16x8_t ov[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int s = s0 + j < p.n_splits ? s0 + j : p.n_splits - 1;  // clamp: duplicates get weight 0 below
-      ml[j] = *reinterpret_cast<const float2*>(p.ws_ml + ((int64_t)s * rows + row) * 2);
-      ov[j] = *reinterpret_cast<const frag_t*>(p.ws_o + ((int64_t)s * rows + row) * DH + dg * 8);
+      ml[j] = *reinterpret_cast<const f32x4_t*>(p.ws_ml + ((int64_t)s * rows + row) * 4);
+      ov[j] = *reinterpret_cast<const f16x8_t*>(p.ws_o + ((int64_t)s * rows + row) * DH + dg * 8);
     }
     float bmax = mmax;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) bmax = fmaxf(bmax, ml[j].x);
+    for (int j = 0; j < 8; ++j) bmax = fmaxf(bmax, ml[j][0]);
     const float carry = bmax > -INFINITY ? __builtin_amdgcn_exp2f(mmax - bmax) : 0.f;  // 0 on the first batch
     den *= carry;
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[j] *= carry;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const float w = (s0 + j < p.n_splits && ml[j].y > 0.f) ? __builtin_amdgcn_exp2f(ml[j].x - bmax) * ml[j].y : 0.f;
+      const float w = (s0 + j < p.n_splits && ml[j][1] > 0.f) ? __builtin_amdgcn_exp2f(ml[j][0] - bmax) * ml[j][1] : 0.f;
       den += w;
+      const float wr = w * ml[j][2];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] += w * (float)ov[j][e];
+      for (int e = 0; e < 8; ++e) acc[e] += wr * (float)ov[j][e];
     }
     mmax = bmax;
   }

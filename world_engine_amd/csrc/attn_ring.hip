@@ -46,6 +46,12 @@
 #include "we_kernels.h"
 #include "../../include/we_attn.h"
 
+#include <atomic>
+
+#ifndef WE_SHIFT_IN_ACC
+#define WE_SHIFT_IN_ACC 0
+#endif
+
 namespace we {
 
 template <int DH>
@@ -298,18 +304,31 @@ attn_ring_kernel(AttnParams p) {
   float m_ref = -INFINITY, l_run = 0.f;
 
   const f32x16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  const float kDead = 3.0e4f;  // shift of logits that must not count (tiles past the end)
-  // K-side fragment of the shift product: contraction index 0 is one for every key
+  // The logits leave the matrix core already shifted by the running reference exponent of this
+  // lane's query (every lane owns one query column of the transposed scores), in one of two ways:
+  //  * WE_SHIFT_IN_ACC: the first product of a block accumulates onto a register block that holds
+  //    -m_ref in all 16 elements; no instruction per block, 16 registers.
+  //  * otherwise: one extra MFMA per block, ones (K side, contraction index 0) x -m_ref (Q side);
+  //    m_ref is kept representable in the element type for that.  8 registers.
+#if WE_SHIFT_IN_ACC
+  f32x16_t shiftv = zero16;
+  auto set_shift = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) shiftv[i] = -m_ref;
+  };
+#else
   frag_t ones_frag = __builtin_bit_cast(frag_t, u32x4_t{0u, 0u, 0u, 0u});
   if (hh == 0) ones_frag[0] = (typename M::elem_t)1.0f;
-  // Q-side fragments: contraction index 0 carries -m_ref of this lane's query, or -kDead
   frag_t shift = __builtin_bit_cast(frag_t, u32x4_t{0u, 0u, 0u, 0u});
-  frag_t dead = shift;
-  if (hh == 0) dead[0] = (typename M::elem_t)(-kDead);
   auto set_shift = [&]() __attribute__((always_inline)) {
     shift = __builtin_bit_cast(frag_t, u32x4_t{0u, 0u, 0u, 0u});
     if (hh == 0) shift[0] = (typename M::elem_t)(-m_ref);
   };
+#endif
+  // Softmax scale: q is multiplied by an exact power of two (no rounding of the element-type
+  // values, so the logits are the exact products' sums), the remaining factor in [1, 2) is
+  // applied to the shifted logits in fp32 inside the exponentials.
+  const float lmul = p.logit_mul;
 
   // probabilities of one 32-key block from its shifted logits: p = 2^(s - sub), packed to the
   // element type; returns this half-wave's share of the row sum (of the rounded values)
@@ -319,7 +338,7 @@ attn_ring_kernel(AttnParams p) {
     for (int m = 0; m < 2; ++m) {
       float e[8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) e[j] = __builtin_amdgcn_exp2f(s[8 * m + j] - sub);
+      for (int j = 0; j < 8; ++j) e[j] = __builtin_amdgcn_exp2f((s[8 * m + j] - sub) * lmul);
       pf[m] = M::pack8(e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7]);
 #pragma unroll
       for (int j = 0; j < 4; ++j) rs = M::add_pair(rs, pf[m], j);
@@ -343,6 +362,11 @@ attn_ring_kernel(AttnParams p) {
   // (two transposing reads each) - running up to 15 reads ahead of the MFMAs.
   frag_t p_prev[2];
   f32x16_t s_cur;
+  // RAGGED only: this wavefront has not seen a key yet (its first block was an empty block of a
+  // short tile), so its reference exponent is a placeholder; cur_keys = keys of the block whose
+  // probabilities the next step computes.
+  bool ref_unset = false;
+  int cur_keys = 32;
   // Fragment registers live across steps: every step starts with its first PRE reads (all K
   // fragments and the first V^T fragment) already in flight, issued during the previous step.
   constexpr int PRE = KS + 2;
@@ -371,8 +395,8 @@ attn_ring_kernel(AttnParams p) {
   // lies past the end of the split)
   // (the K fragments at koff_c were requested by the previous step; the offset documents the call)
   auto step = [&](auto /*koff_c*/, auto voff_c, auto nkoff_c, auto nvoff_c, int nkeys, auto&& mid) __attribute__((always_inline)) {
-    // logits of a block past the end are never consumed; only a short tile's empty block needs them dead
-    const bool live = !RAGGED || nkeys > 0;
+    // (logits of a block past the end of the split are never consumed; a short tile's empty block
+    // is masked after its products)
     // next own V fragment to request / next-step read pairs requested so far
     int vnext = 1, npair = 0;
     constexpr int NPAIR = PRE / 2;            // the next step's first reads go out two at a time
@@ -390,37 +414,46 @@ attn_ring_kernel(AttnParams p) {
     // From here to the end of the product the issue order is pinned statement by statement
     // (sched_barrier): MFMA, the reads that refill the queue, a slice of the VALU work.
     __builtin_amdgcn_sched_barrier(0);
-    f32x16_t s_next = M::mma(ones_frag, live ? shift : dead, zero16);
     frag_t p_cur[2];
     float e[16];
     float rs = 0.f;
     // VALU slices: the 16 exponentials of the current block are spread evenly over the MFMAs of
-    // the step (slot 0 follows the shift product, slots 1..KS the logits, the rest the product).
-    // The two wavefronts of a SIMD run in phase, so bunching them under the logits would saturate
-    // the quarter-rate unit there and leave it idle under the product.
+    // the step.  The two wavefronts of a SIMD run in phase, so bunching them under the logits
+    // would saturate the quarter-rate unit there and leave it idle under the product.
     constexpr int EPS = 16 / (KS + NV);
     static_assert(EPS * (KS + NV) == 16, "exponentials per slot");
     auto exp_slot = [&](int g) __attribute__((always_inline)) {
 #pragma unroll
       for (int t = 0; t < EPS; ++t)
         if (g * EPS + t < 16) {
-          e[g * EPS + t] = __builtin_amdgcn_exp2f(s_cur[g * EPS + t]);
+          e[g * EPS + t] = __builtin_amdgcn_exp2f(s_cur[g * EPS + t] * lmul);
           // an exponential has no side effect, so nothing else keeps it in its slot: left alone the
           // compiler sinks the first nine of a step below the tile DMAs
           asm volatile("" : "+v"(e[g * EPS + t]));
         }
     };
+#if WE_SHIFT_IN_ACC
+    constexpr int S0 = 0;   // slot of the exponentials that follow the first logits product
+    f32x16_t s_next;
+#else
+    constexpr int S0 = 1;   // slot 0 follows the shift product
+    f32x16_t s_next = M::mma(ones_frag, shift, zero16);
     exp_slot(0);
     __builtin_amdgcn_sched_barrier(0);
+#endif
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
+#if WE_SHIFT_IN_ACC
+      s_next = M::mma(__builtin_bit_cast(frag_t, kf[ks]), qf[ks], ks == 0 ? shiftv : s_next);
+#else
       s_next = M::mma(__builtin_bit_cast(frag_t, kf[ks]), qf[ks], s_next);
+#endif
       // keep the read queue full without exceeding the 15 reads the counter can track
       if (vnext < NV && ks <= 12 - KS) {
         read_v(voff_c, vnext);
         ++vnext;
         }
-      exp_slot(1 + ks);
+      exp_slot(S0 + ks);
       __builtin_amdgcn_sched_barrier(0);
     }
     mid();  // the tile DMAs of this iteration go out here, under the MFMAs already queued
@@ -436,7 +469,7 @@ attn_ring_kernel(AttnParams p) {
       o[i % DB] = M::mma(__builtin_bit_cast(frag_t, a4), p_prev[i / DB], o[i % DB]);
       if (i >= I0 && npair < NPAIR) next_pair();
       // VALU slices: the last exponentials; packing of the two 16-key halves and their row sums
-      exp_slot(1 + KS + i);
+      exp_slot(S0 + KS + i);
       if (i == 1) p_cur[0] = M::pack8(e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7]);
       if (i == 2) {
 #pragma unroll
@@ -448,15 +481,20 @@ attn_ring_kernel(AttnParams p) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) rs = M::add_pair(rs, p_cur[1], t);
 
-    if (__ballot(!(rs <= 256.f)) != 0ull) {
+    // first block with keys of a wavefront that started on an empty block: nothing is accumulated
+    // yet, so the placeholder reference is replaced by this block's own maximum, up or down
+    // (a placeholder far above every real logit would make all of them underflow to zero)
+    const bool seed = RAGGED && ref_unset && cur_keys > 0;
+    if (seed || __ballot(!(rs <= 256.f)) != 0ull) {
       // Rare: some probability of this block may exceed 2^8.  Raise the reference of the rows
       // that need it, redo the block's probabilities exactly, re-base the logits of the next
       // block, which were produced with the old reference, and rescale the accumulators: they hold
       // the blocks before this one (the last of those products was issued above).
       const float mx = block_max(s_cur);
-      const float m_new = mx > 0.f ? M::round_up(m_ref + mx) : m_ref;
+      const float m_new = (seed ? mx > -INFINITY : mx > 0.f) ? M::round_up(m_ref + mx) : m_ref;
       const float delta = m_new - m_ref;
-      const float alpha = __builtin_amdgcn_exp2f(-delta);
+      const float alpha = seed ? 1.f : __builtin_amdgcn_exp2f(-delta * lmul);  // seed: sums and accumulators are still zero
+      if (RAGGED) ref_unset = false;
       rs = probabilities(p_cur, s_cur, delta);
       l_run *= alpha;
       m_ref = m_new;
@@ -471,7 +509,8 @@ attn_ring_kernel(AttnParams p) {
     l_run += rs;
     p_prev[0] = p_cur[0];
     p_prev[1] = p_cur[1];
-    if (RAGGED && nkeys > 0 && nkeys < 32) mask_keys(s_next, nkeys);  // short last tile of a slot
+    if (RAGGED && nkeys < 32) mask_keys(s_next, nkeys);  // short last tile of a slot (or an empty block of it)
+    if (RAGGED) cur_keys = nkeys;
     s_cur = s_next;
   };
 
@@ -513,9 +552,9 @@ attn_ring_kernel(AttnParams p) {
       }
       dma_v(o1, 1);
     }
-    // ---- Q stays in registers for the whole kernel, pre-multiplied by scale*log2(e); done while
-    //      the first tiles are on their way ----
-    const float c2 = p.scale_log2;
+    // ---- Q stays in registers for the whole kernel, multiplied by a power of two (exact); done
+    //      while the first tiles are on their way ----
+    const float c2 = p.q_pow2;
   #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const frag_t raw = qf[ks];
@@ -536,6 +575,10 @@ attn_ring_kernel(AttnParams p) {
       if (RAGGED && nk0 < 32) mask_keys(s_cur, nk0);
       const float mx0 = block_max(s_cur);
       m_ref = mx0 > -INFINITY ? M::round_up(mx0) : 0.f;  // (a block of the first tile may be empty)
+      if (RAGGED) {
+        ref_unset = nk0 == 0;
+        cur_keys = nk0;
+      }
       set_shift();
 #pragma unroll
       for (int i = 0; i < 16; ++i) s_cur[i] -= m_ref;
@@ -618,6 +661,7 @@ attn_ring_kernel(AttnParams p) {
   float lo, up;
   half_wave_pair(l_run, lo, up);
   float l_tot = lo + up;
+  m_ref *= lmul;  // from the matrix core's units (logits / lmul) to the log2 domain the merges work in
 
   if (KSPLIT == 2) {
     // ---- the two wavefronts of a query block merge their (m, l, O) through LDS ----
@@ -635,7 +679,10 @@ attn_ring_kernel(AttnParams p) {
     __syncthreads();
     if (hb == 1) return;
     const f32x4_t ml1 = mb[(DB * 4) * 64];
-    const float m1 = ml1[0], l1 = ml1[1];
+    // a wavefront whose sum is zero saw no key (or only keys that vanish against its reference):
+    // its reference must not take part in the maximum
+    const float m1 = ml1[1] > 0.f ? ml1[0] : -INFINITY, l1 = ml1[1];
+    if (!(l_tot > 0.f)) m_ref = -INFINITY;
     const float mm = fmaxf(m_ref, m1);
     if (mm > -INFINITY) {
       const float a0 = __builtin_amdgcn_exp2f(m_ref - mm), a1 = __builtin_amdgcn_exp2f(m1 - mm);
@@ -660,9 +707,23 @@ attn_ring_kernel(AttnParams p) {
   float gate_v = 1.f;
   if (p.gate != nullptr && nsp == 1 && qrow < p.T)
     gate_v = (float)reinterpret_cast<const typename M::elem_t*>(p.gate)[b * p.gs_b + h * p.gs_h + (int64_t)qrow * p.gs_t];
-  if (nsp > 1 && valid && hh == 0) {
-    float2 ml = make_float2(m_ref, l_tot);
-    *reinterpret_cast<float2*>(p.ws_ml + ((int64_t)split * rows + (row - p.ws_row0)) * 2) = ml;
+  // A split leaves its partial output as fp16 values in [-1, 1] plus one fp32 scale per row (the
+  // row's largest normalised magnitude): 11 significant bits whatever the element type, for the
+  // bytes of a bf16 row, and no overflow whatever V holds.
+  float mul = inv;
+  if (nsp > 1) {
+    float amax = 0.f;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(o[db][i]));
+    float alo, aup;
+    half_wave_pair(amax, alo, aup);
+    amax = fmaxf(alo, aup);
+    mul = amax > 0.f ? 1.f / amax : 0.f;
+    if (valid && hh == 0)
+      *reinterpret_cast<f32x4_t*>(p.ws_ml + ((int64_t)split * rows + (row - p.ws_row0)) * 4) =
+          f32x4_t{l_tot > 0.f ? m_ref : -INFINITY, l_tot, amax * inv, 0.f};
   }
 #pragma unroll
   for (int db = 0; db < DB; ++db) {
@@ -673,8 +734,8 @@ attn_ring_kernel(AttnParams p) {
       float f[8];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(o[db][4 * c + e] * inv),
-                                                  __float_as_uint(o[db][4 * c + 4 + e] * inv), false, false);
+        auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(o[db][4 * c + e] * mul),
+                                                  __float_as_uint(o[db][4 * c + 4 + e] * mul), false, false);
         f[e] = __uint_as_float(r[0]);
         f[4 + e] = __uint_as_float(r[1]);
       }
@@ -691,7 +752,7 @@ attn_ring_kernel(AttnParams p) {
           *reinterpret_cast<frag_t*>(dst) = y;
         } else {
           uint16_t* dst = p.ws_o + ((int64_t)split * rows + (row - p.ws_row0)) * DH + d0;
-          *reinterpret_cast<frag_t*>(dst) = M::pack8(f[0], f[1], f[2], f[3], f[4], f[5], f[6], f[7]);
+          *reinterpret_cast<f16x8_t*>(dst) = F16Mma::pack8(f[0], f[1], f[2], f[3], f[4], f[5], f[6], f[7]);
         }
       }
     }
@@ -702,16 +763,16 @@ template <typename M, int DH, int KSPLIT, bool RAGGED>
 static hipError_t launch_ring_r(const AttnParams& p, hipStream_t stream) {
   // the LDS limit of a kernel is a per-device setting: raise it once on every device that launches
   // (a flag that two threads both find unset is set twice, which is harmless)
-  static bool configured[64] = {};
+  static std::atomic<bool> configured[64] = {};
   const int lds = RingLds<DH>::kBytes;
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
-  if (dev < 0 || dev >= 64 || !configured[dev]) {
+  if (dev < 0 || dev >= 64 || !configured[dev].load(std::memory_order_acquire)) {
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_ring_kernel<M, DH, KSPLIT, RAGGED>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     if (e != hipSuccess) return e;
-    if (dev >= 0 && dev < 64) configured[dev] = true;
+    if (dev >= 0 && dev < 64) configured[dev].store(true, std::memory_order_release);
   }
   const int rounds = (p.unit_splits + 7) / 8;
   const dim3 grid((unsigned)(8 * p.q_tiles), (unsigned)p.group, (unsigned)rounds);
@@ -723,15 +784,27 @@ static hipError_t launch_ring_t(const AttnParams& p, hipStream_t stream) {
   return p.T % BN == 0 ? launch_ring_r<M, DH, KSPLIT, false>(p, stream) : launch_ring_r<M, DH, KSPLIT, true>(p, stream);
 }
 
-hipError_t launch_attn_ring(const AttnParams& p, int Dh, int dtype, int ksplit, hipStream_t stream) {
-  if (dtype == WE_DTYPE_BF16) {
-    if (Dh == 128) return ksplit == 2 ? launch_ring_t<Bf16Mma, 128, 2>(p, stream) : launch_ring_t<Bf16Mma, 128, 1>(p, stream);
-    if (Dh == 64) return ksplit == 2 ? launch_ring_t<Bf16Mma, 64, 2>(p, stream) : launch_ring_t<Bf16Mma, 64, 1>(p, stream);
-  } else if (dtype == WE_DTYPE_F16) {
-    if (Dh == 128) return ksplit == 2 ? launch_ring_t<F16Mma, 128, 2>(p, stream) : launch_ring_t<F16Mma, 128, 1>(p, stream);
-    if (Dh == 64) return ksplit == 2 ? launch_ring_t<F16Mma, 64, 2>(p, stream) : launch_ring_t<F16Mma, 64, 1>(p, stream);
-  }
-  return hipErrorInvalidValue;
+// The four (element type, head dim) families are compiled as separate objects (WE_RING_PART selects
+// one; undefined = all of them in this translation unit) so that they build in parallel.
+#if !defined(WE_RING_PART) || WE_RING_PART == 0
+hipError_t launch_attn_ring_bf16_128(const AttnParams& p, int ksplit, hipStream_t stream) {
+  return ksplit == 2 ? launch_ring_t<Bf16Mma, 128, 2>(p, stream) : launch_ring_t<Bf16Mma, 128, 1>(p, stream);
 }
+#endif
+#if !defined(WE_RING_PART) || WE_RING_PART == 1
+hipError_t launch_attn_ring_bf16_64(const AttnParams& p, int ksplit, hipStream_t stream) {
+  return ksplit == 2 ? launch_ring_t<Bf16Mma, 64, 2>(p, stream) : launch_ring_t<Bf16Mma, 64, 1>(p, stream);
+}
+#endif
+#if !defined(WE_RING_PART) || WE_RING_PART == 2
+hipError_t launch_attn_ring_f16_128(const AttnParams& p, int ksplit, hipStream_t stream) {
+  return ksplit == 2 ? launch_ring_t<F16Mma, 128, 2>(p, stream) : launch_ring_t<F16Mma, 128, 1>(p, stream);
+}
+#endif
+#if !defined(WE_RING_PART) || WE_RING_PART == 3
+hipError_t launch_attn_ring_f16_64(const AttnParams& p, int ksplit, hipStream_t stream) {
+  return ksplit == 2 ? launch_ring_t<F16Mma, 64, 2>(p, stream) : launch_ring_t<F16Mma, 64, 1>(p, stream);
+}
+#endif
 
 }  // namespace we

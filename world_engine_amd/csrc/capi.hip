@@ -3,6 +3,8 @@
 #include "../../include/we_attn.h"
 #include "we_kernels.h"
 
+#include <cmath>
+
 namespace {
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -146,7 +148,7 @@ int prepare_attn(const void* q, const int64_t* q_strides, const void* kv, const 
     return WE_ERR_ALIGNMENT;
 
   pl = plan_attn(B, H, Hkv, T, L, n_splits, variant_of(q_tile));
-  const size_t ws_need = (size_t)pl.n_splits * (size_t)pl.ws_rows * ((size_t)Dh * 2 + 2 * sizeof(float));
+  const size_t ws_need = (size_t)pl.n_splits * (size_t)pl.ws_rows * ((size_t)Dh * 2 + 4 * sizeof(float));
   if (ws_need > 0) {
     if (!workspace || !aligned16(workspace)) return WE_ERR_WORKSPACE;
     if (workspace_bytes < ws_need) return WE_ERR_WORKSPACE;
@@ -167,7 +169,13 @@ int prepare_attn(const void* q, const int64_t* q_strides, const void* kv, const 
   p.group = H / Hkv;
   p.members = p.group * p.q_tiles;
   p.unit_splits = pl.units_whole + (B * Hkv - pl.units_whole) * pl.n_splits;
-  p.scale_log2 = scale * 1.4426950408889634f;
+  {
+    const float c2 = scale * 1.4426950408889634f;
+    int ex = 0;
+    const float mant = frexpf(c2, &ex);       // c2 = mant * 2^ex, mant in [0.5, 1)
+    p.q_pow2 = ldexpf(1.f, ex - 1);
+    p.logit_mul = mant * 2.f;
+  }
   p.gate = nullptr; p.gs_b = p.gs_h = p.gs_t = 0;
 
   if ((p.unit_splits + 7) / 8 > 65535 || p.group > 65535 || (int64_t)B * H - (int64_t)pl.units_whole * p.group > 65535)
@@ -177,7 +185,11 @@ int prepare_attn(const void* q, const int64_t* q_strides, const void* kv, const 
 
 int launch_attn(const we::AttnParams& p, const AttnPlan& pl, int Dh, int dtype, hipStream_t st) {
   if (dtype == WE_DTYPE_F32) return we::launch_attn_ring_f32(p, Dh, st) == hipSuccess ? WE_OK : WE_ERR_LAUNCH;
-  if (we::launch_attn_ring(p, Dh, dtype, pl.variant == 1 ? 2 : 1, st) != hipSuccess) return WE_ERR_LAUNCH;
+  const int ksplit = pl.variant == 1 ? 2 : 1;
+  hipError_t e;
+  if (dtype == WE_DTYPE_BF16) e = Dh == 128 ? we::launch_attn_ring_bf16_128(p, ksplit, st) : we::launch_attn_ring_bf16_64(p, ksplit, st);
+  else e = Dh == 128 ? we::launch_attn_ring_f16_128(p, ksplit, st) : we::launch_attn_ring_f16_64(p, ksplit, st);
+  if (e != hipSuccess) return WE_ERR_LAUNCH;
   if (pl.n_splits > 1 && we::launch_attn_combine(p, Dh, dtype, st) != hipSuccess) return WE_ERR_LAUNCH;
   return WE_OK;
 }
@@ -258,7 +270,7 @@ size_t we_attn_workspace_bytes(int32_t B, int32_t H, int32_t Hkv, int32_t T, int
   const int variant = variant_of(q_tile);
   if (variant < 0) return 0;
   const AttnPlan pl = plan_attn(B, H, Hkv, T, L, n_splits, variant);
-  return (size_t)pl.n_splits * (size_t)pl.ws_rows * ((size_t)Dh * 2 + 2 * sizeof(float));
+  return (size_t)pl.n_splits * (size_t)pl.ws_rows * ((size_t)Dh * 2 + 4 * sizeof(float));
 }
 
 int we_attn_ring_fwd(const void* q, const int64_t q_strides[3], const void* kv, const uint8_t* written,

@@ -41,8 +41,8 @@ struct AttnParams {
   const uint8_t* written;
   const int64_t* t_pos;
   void* out;
-  uint16_t* ws_o;  // [n_splits][rows >= ws_row0][Dh] normalised partial outputs, element type
-  float* ws_ml;    // [n_splits][rows >= ws_row0][2]  softmax reference (log2 domain) and sum
+  uint16_t* ws_o;  // [n_splits][rows >= ws_row0][Dh] normalised partial outputs / row scale, fp16 in [-1, 1]
+  float* ws_ml;    // [n_splits][rows >= ws_row0][4]  softmax reference (log2 domain), sum, row scale, unused
   int64_t qs_b, qs_h, qs_t;
   int64_t os_b, os_h, os_t;
   int64_t L;
@@ -55,7 +55,9 @@ struct AttnParams {
   int group;        // query heads per kv head, H / Hkv
   int members;      // workgroups that share one K/V stream: group * q_tiles
   int unit_splits;  // units_whole + (B * Hkv - units_whole) * n_splits
-  float scale_log2; // softmax scale * log2(e)
+  // softmax scale * log2(e) = q_pow2 * logit_mul: q is multiplied by q_pow2, a power of two (exact in
+  // the element type), the logits by logit_mul in [1, 2) in fp32
+  float q_pow2, logit_mul;
   // optional per (batch, head, token) output gate, element type (src/model/attn.py:117-119)
   const void* gate;
   int64_t gs_b, gs_h, gs_t;
@@ -63,8 +65,12 @@ struct AttnParams {
 
 hipError_t launch_rope_kv_store(const StoreParams& p, int dtype, hipStream_t stream);
 
-// main kernel: ksplit = 2 -> 128 queries per workgroup, 1 -> 256
-hipError_t launch_attn_ring(const AttnParams& p, int Dh, int dtype, int ksplit, hipStream_t stream);
+// main kernel, one launcher per (element type, head dim) family: ksplit = 2 -> 128 queries per
+// workgroup, 1 -> 256
+hipError_t launch_attn_ring_bf16_128(const AttnParams& p, int ksplit, hipStream_t stream);
+hipError_t launch_attn_ring_bf16_64(const AttnParams& p, int ksplit, hipStream_t stream);
+hipError_t launch_attn_ring_f16_128(const AttnParams& p, int ksplit, hipStream_t stream);
+hipError_t launch_attn_ring_f16_64(const AttnParams& p, int ksplit, hipStream_t stream);
 // fp32 caches: plain vector-ALU kernel, one pass, no context splitting
 hipError_t launch_attn_ring_f32(const AttnParams& p, int Dh, hipStream_t stream);
 hipError_t launch_attn_combine(const AttnParams& p, int Dh, int dtype, hipStream_t stream);
