@@ -41,8 +41,12 @@ extern "C" {
 #define WE_ERR_ALIGNMENT (-4)     /* pointer or stride not 16-byte aligned */
 #define WE_ERR_WORKSPACE (-5)     /* split-context workspace missing or too small */
 #define WE_ERR_LAUNCH (-6)        /* the HIP runtime refused the launch */
+#define WE_ERR_SCRATCH_LIMIT (-7) /* we_attn_ring_fwd_static: sizes need more scratch than WE_STATIC_SCRATCH_BYTES */
 
 #define WE_MAX_SLOTS 256 /* maximum number of ring slots L / T */
+
+/* size of the library's own split-context scratch buffer (see we_attn_ring_fwd_static) */
+#define WE_STATIC_SCRATCH_BYTES (32u << 20)
 
 /* Library version: major*10000 + minor*100 + patch. */
 int we_version(void);
@@ -154,6 +158,29 @@ int we_attn_ring_fwd(const void* q, const int64_t q_strides[3],
                      int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L,
                      int32_t dilation, float scale, int32_t n_splits, int32_t q_tile,
                      int32_t dtype, void* stream);
+
+/*
+ * we_attn_ring_fwd for callers that cannot allocate device memory, not even a workspace: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference (whose attention call allocates through torch as it pleases).
+ * Arguments, requirements and results are those of we_attn_ring_fwd, bit for bit, without the
+ * workspace pair: the split-context partial results go to a buffer of WE_STATIC_SCRATCH_BYTES that
+ * is part of the library's device image (every GPU the library runs on holds one copy until the
+ * process ends; its address is looked up once per device, on the first call made with that
+ * device current).  Sizes whose we_attn_workspace_bytes(...) exceeds WE_STATIC_SCRATCH_BYTES are
+ * rejected with WE_ERR_SCRATCH_LIMIT and nothing is launched.  The call itself performs no
+ * hipMalloc / hipFree and calls no allocating library routine.
+ * All calls on one GPU share that GPU's buffer: calls that overlap in time on one GPU (different
+ * streams, or parallel branches of one graph) race on it; calls that follow each other on a
+ * stream do not.  Nothing in the buffer has to start at zero (every partial row a call reads was
+ * written by that call's first kernel).
+ */
+int we_attn_ring_fwd_static(const void* q, const int64_t q_strides[3],
+                            const void* kv, const uint8_t* written, const int64_t* t_pos,
+                            void* out, const int64_t out_strides[3],
+                            int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L,
+                            int32_t dilation, float scale, int32_t n_splits, int32_t q_tile,
+                            int32_t dtype, void* stream);
 
 /*
  * Optional work of the reference's attention module that sits right in front of and right behind

@@ -14,6 +14,8 @@ LIB_PATH = os.path.join(_HERE, "libwe_attn.so")
 
 WE_DTYPE_BF16, WE_DTYPE_F16, WE_DTYPE_F32 = 0, 1, 2
 WE_MAX_SLOTS = 256
+WE_STATIC_SCRATCH_BYTES = 32 << 20
+WE_ERR_SCRATCH_LIMIT = -7
 
 _I64x3 = POINTER(c_int64)
 
@@ -53,6 +55,13 @@ SIGNATURES = {
         c_void_p, c_void_p, c_void_p,              # kv, written, t_pos
         c_void_p, _I64x3,                          # out, out_strides
         c_void_p, c_size_t,                        # workspace, bytes
+        c_int32, c_int32, c_int32, c_int32, c_int32, c_int64,   # B H Hkv T Dh L
+        c_int32, c_float, c_int32, c_int32, c_int32, c_void_p,  # dilation scale n_splits q_tile dtype stream
+    ]),
+    "we_attn_ring_fwd_static": (c_int32, [
+        c_void_p, _I64x3,                          # q, q_strides
+        c_void_p, c_void_p, c_void_p,              # kv, written, t_pos
+        c_void_p, _I64x3,                          # out, out_strides
         c_int32, c_int32, c_int32, c_int32, c_int32, c_int64,   # B H Hkv T Dh L
         c_int32, c_float, c_int32, c_int32, c_int32, c_void_p,  # dilation scale n_splits q_tile dtype stream
     ]),

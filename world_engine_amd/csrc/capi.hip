@@ -4,8 +4,33 @@
 #include "we_kernels.h"
 
 #include <cmath>
+#include <mutex>
+
+// Split-context partial results of we_attn_ring_fwd_static: part of the library's device image, so
+// that the entry point needs no allocation and no caller-owned workspace.  Every GPU the library
+// runs on holds its own copy at its own address; host code must never use the array's name as an
+// address (on the host it is a stand-in for the symbol), only what hipGetSymbolAddress returns
+// with the device in question current.
+static __device__ __align__(256) unsigned char scratch[WE_STATIC_SCRATCH_BYTES];
 
 namespace {
+
+// Device address of `scratch` on the current device, looked up once per device.
+int static_scratch(void** out) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex mu;
+  static void* ptr[kMaxDevices] = {};
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return WE_ERR_LAUNCH;
+  std::lock_guard<std::mutex> lock(mu);
+  if (ptr[dev] == nullptr) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) return WE_ERR_LAUNCH;
+    ptr[dev] = p;
+  }
+  *out = ptr[dev];
+  return WE_OK;
+}
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -209,6 +234,7 @@ const char* we_error_string(int code) {
     case WE_ERR_ALIGNMENT: return "pointer or stride breaks 16-byte alignment";
     case WE_ERR_WORKSPACE: return "split-context workspace missing or too small";
     case WE_ERR_LAUNCH: return "HIP runtime refused the kernel launch";
+    case WE_ERR_SCRATCH_LIMIT: return "sizes need more split-context scratch than the library's static buffer (WE_STATIC_SCRATCH_BYTES) holds";
     default: return "unknown error code";
   }
 }
@@ -285,6 +311,29 @@ int we_attn_ring_fwd(const void* q, const int64_t q_strides[3], const void* kv, 
   if (rc != WE_OK) return rc;
   hipStream_t st = static_cast<hipStream_t>(stream);
   return launch_attn(p, pl, Dh, dtype, st);
+}
+
+int we_attn_ring_fwd_static(const void* q, const int64_t q_strides[3], const void* kv, const uint8_t* written,
+                            const int64_t* t_pos, void* out, const int64_t out_strides[3], int32_t B, int32_t H,
+                            int32_t Hkv, int32_t T, int32_t Dh, int64_t L, int32_t dilation, float scale,
+                            int32_t n_splits, int32_t q_tile, int32_t dtype, void* stream) {
+  // sizes first, so that a call that cannot fit is refused before anything else happens
+  if (B > 0 && H > 0 && Hkv > 0 && H % Hkv == 0 && T > 0 && Dh > 0 && L > 0 && n_splits >= 0 && variant_of(q_tile) >= 0 &&
+      dtype != WE_DTYPE_F32) {
+    const AttnPlan sz = plan_attn(B, H, Hkv, T, L, n_splits, variant_of(q_tile));
+    const unsigned long long need =
+        (unsigned long long)sz.n_splits * (unsigned long long)sz.ws_rows * ((unsigned long long)Dh * 2 + 4 * sizeof(float));
+    if (need > WE_STATIC_SCRATCH_BYTES) return WE_ERR_SCRATCH_LIMIT;
+  }
+  void* ws = nullptr;
+  int rc = static_scratch(&ws);
+  if (rc != WE_OK) return rc;
+  we::AttnParams p;
+  AttnPlan pl;
+  rc = prepare_attn(q, q_strides, kv, written, t_pos, out, out_strides, ws, WE_STATIC_SCRATCH_BYTES, B, H, Hkv, T, Dh,
+                    L, dilation, scale, n_splits, q_tile, dtype, p, pl);
+  if (rc != WE_OK) return rc;
+  return launch_attn(p, pl, Dh, dtype, static_cast<hipStream_t>(stream));
 }
 
 int we_rope_kv_attn_fwd(const void* q, const void* k, const void* v, const int64_t q_strides[3],

@@ -207,6 +207,37 @@ def attn_ring(q: Tensor, kv: Tensor, written: Tensor, t_pos: Tensor, L: int, dil
     return out
 
 
+def attn_ring_static(q: Tensor, kv: Tensor, written: Tensor, t_pos: Tensor, L: int, dilation: int, out: Tensor,
+                     scale: Optional[float] = None, n_splits: int = 0, q_tile: int = 0) -> Tensor:
+    """``attn_ring`` through ``we_attn_ring_fwd_static``: no workspace argument and no allocation
+    anywhere (``out`` must be given); the split-context partial results go to a buffer inside the
+    library's device image (``_capi.WE_STATIC_SCRATCH_BYTES``).  Sizes that need more raise.  Calls
+    that overlap on one GPU race on that buffer.  No counterpart in the reference; for callers
+    that cannot allocate."""
+    dev = _need_device(q, kv, written, t_pos, out)
+    if q.dim() != 4:
+        raise RuntimeError("q must be [B, H, T, Dh]")
+    B, H, T, Dh = q.shape
+    if kv.dim() != 5 or kv.shape[0] != 2 or kv.shape[1] != B or kv.shape[3] != L + T or kv.shape[4] != Dh:
+        raise RuntimeError("kv must be [2, B, Hkv, L+T, Dh] matching q")
+    if not kv.is_contiguous() or kv.dtype != q.dtype:
+        raise RuntimeError("kv must be contiguous and of q's element type")
+    if written.dtype != torch.bool or written.numel() != L + T or not written.is_contiguous():
+        raise RuntimeError("written must be a contiguous bool [L+T] tensor")
+    if t_pos.dtype != torch.long or t_pos.numel() < 1:
+        raise RuntimeError("t_pos must be a non-empty int64 tensor")
+    if tuple(out.shape) != (B, H, T, Dh) or out.dtype != q.dtype:
+        raise RuntimeError("out must be [B, H, T, Dh] of q's element type on q's device")
+    scale = 1.0 / math.sqrt(Dh) if scale is None else float(scale)
+    with torch.cuda.device(dev):     # the buffer's address is per device: the call must see q's device as current
+        code = _capi.lib().we_attn_ring_fwd_static(
+            q.data_ptr(), _bhtd_strides(q, "q"), kv.data_ptr(), written.data_ptr(), t_pos.data_ptr(),
+            out.data_ptr(), _bhtd_strides(out, "out"), B, H, kv.shape[2], T, Dh, L, dilation, scale, n_splits, q_tile,
+            _dtype_code(q), _stream_ptr(dev))
+    _capi.check(code, "we_attn_ring_fwd_static")
+    return out
+
+
 def rope_kv_attn(q: Tensor, k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor], cos_table: Tensor,
                  sin_table: Tensor, grid_h: int, grid_w: int, kv: Tensor, written: Tensor, L: int,
                  dilation: int, is_frozen: bool, scale: Optional[float] = None, n_splits: int = 0,
