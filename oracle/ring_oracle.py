@@ -14,7 +14,9 @@ Reference sources followed (paths relative to the world_engine checkout):
 * ``src/model/kv_cache.py:12-61``   meaning of the block mask: key j is visible iff mask[j]
 * ``src/model/kv_cache.py:157-193`` per-layer window/dilation choice, frozen flag, k/v stacking
 * ``src/model/attn.py:22-40``       table-driven RoPE (fp32 math, de-interleaved output)
-* ``src/model/attn.py:99-122`` / ``src/patch_model.py:116-141``  order of operations
+* ``src/model/attn.py:99-122`` / ``src/patch_model.py:116-141``  order of operations, incl. the
+  module's element-wise steps around the path: value-residual lerp (``attn.py:105-107``), weightless
+  QK RMS norm (``attn.py:109``, ``src/model/nn.py:55-56``), sigmoid head gate (``attn.py:117-119``)
 * ``src/world_engine.py:139-152``   frozen denoise passes followed by one unfrozen cache pass
 * ``torch/_higher_order_ops/flex_attention.py:159-267`` (torch 2.10, third-party) dtype flow
   of eager ``flex_attention``: fp32 scores, ``* scale``, ``where(mask, s, -inf)``, softmax,
@@ -32,6 +34,9 @@ Pinning status (see tests/test_oracle_pins.py; the reference ships no tests or g
 * ``attention_reference_path`` / ``attention_fp32``  pinned: torch's own eager
   ``flex_attention`` with a ``BlockMask.from_kv_blocks`` mask (library routine), SDPA on the
   gathered visible keys, key-permutation invariance, fp64 brute force
+* ``rms_norm`` / ``value_lerp`` / ``gate_output``  pinned: torch's own ``F.rms_norm`` / ``torch.lerp``
+  (library routines, the calls the reference makes) bit for bit on the CPU, plus closed cases
+  (unit RMS, power-of-two scale invariance, lerp end points, gate 0 / 1)
 * ``rope_table_1d``                  synthetic table of the benchmark configurations (not a
   reference function); checked against direct fp64 evaluation
 * ``ortho_rope_table``               parity unpinned: depends on ``rotary_embedding_torch``
@@ -281,20 +286,68 @@ def attention_fp32(q: Tensor, k_all: Tensor, v_all: Tensor, mask: Tensor,
 
 
 # --------------------------------------------------------------------------------------
+# the module's element-wise steps around the path
+#                     src/model/attn.py:105-109,117-119, src/model/nn.py:55-56
+# --------------------------------------------------------------------------------------
+def rms_norm(x: Tensor, eps: Optional[float] = None) -> Tensor:
+    """Weightless RMS norm over the last dimension, ``F.rms_norm(x, (x.size(-1),))``
+    (src/model/nn.py:55-56): ``x / sqrt(mean(x^2) + eps)`` evaluated in fp32 for low-precision
+    inputs and rounded to ``x``'s dtype.  torch's default epsilon is the machine epsilon of the
+    arithmetic type, i.e. fp32's for bf16 / f16 / fp32 inputs."""
+    wp = torch.float64 if x.dtype == torch.float64 else torch.float32
+    if eps is None:
+        eps = torch.finfo(wp).eps
+    xf = x.to(wp)
+    ms = xf.pow(2).mean(dim=-1, keepdim=True)
+    return (xf * torch.rsqrt(ms + eps)).to(x.dtype)
+
+
+def value_lerp(v: Tensor, v1: Tensor, weight: Tensor) -> Tensor:
+    """Value residual ``torch.lerp(v, v1, weight)`` (src/model/attn.py:105-107): fp32 arithmetic for
+    low-precision tensors, ``v + w (v1 - v)`` below ``w = 0.5`` and ``v1 - (v1 - v)(1 - w)`` from
+    there on (the formula torch switches between to stay monotonic), rounded to ``v``'s dtype."""
+    wp = torch.float64 if v.dtype == torch.float64 else torch.float32
+    a, b = v.to(wp), v1.to(wp)
+    w = weight.to(wp)
+    d = b - a
+    out = torch.where(w.abs() < 0.5, a + w * d, b - d * (1 - w))
+    return out.to(v.dtype)
+
+
+def gate_output(y: Tensor, gates: Tensor) -> Tensor:
+    """Head gate (src/model/attn.py:117-119): ``y * gates.permute(0, 2, 1).unsqueeze(-1)`` with
+    ``y`` ``[B,H,T,Dh]`` and ``gates`` ``[B,T,H]`` (sigmoid already applied), a product of two
+    tensors of the element type, rounded to it."""
+    return y * gates.permute(0, 2, 1).unsqueeze(-1)
+
+
+# --------------------------------------------------------------------------------------
 # one attention-layer step in the reference's order of operations
-#                                  src/model/attn.py:105-116, src/patch_model.py:128-133
+#                                  src/model/attn.py:105-119, src/patch_model.py:124-137
 # --------------------------------------------------------------------------------------
 def layer_step(cache: OracleStaticKVCache, layer: int, q: Tensor, k: Tensor, v: Tensor,
                pos_ids: Dict[str, Tensor], cos_table: Tensor, sin_table: Tensor,
                height: int, width: int, scale: Optional[float] = None,
-               reference_dtype_flow: bool = True) -> Tuple[Tensor, Tensor]:
-    """RoPE(q), RoPE(k) -> cache upsert -> masked attention.  Returns ``(out, q_rot)``."""
+               reference_dtype_flow: bool = True, qk_norm: bool = False,
+               v1: Optional[Tensor] = None, v_lamb: Optional[Tensor] = None,
+               gates: Optional[Tensor] = None) -> Tuple[Tensor, Tensor]:
+    """[lerp(v, v1, v_lamb)] -> [rms_norm(q), rms_norm(k)] -> RoPE(q), RoPE(k) -> cache upsert ->
+    masked attention -> [gate].  The bracketed steps are the module's optional ones and are off
+    by default.  Returns ``(out, q_rot)``; with ``reference_dtype_flow=False`` the attention (and
+    the gate multiply) are evaluated in fp32 on the element-type inputs."""
+    if v1 is not None:
+        v = value_lerp(v, v1.view_as(v), v_lamb)
+    if qk_norm:
+        q, k = rms_norm(q), rms_norm(k)
     cos, sin = rope_angles(pos_ids, cos_table, sin_table, height, width)
     q_rot = rope_apply(q, cos, sin)
     k_rot = rope_apply(k, cos, sin)
     k_all, v_all, mask = cache.upsert(k_rot, v, pos_ids, layer)
     fn = attention_reference_path if reference_dtype_flow else attention_fp32
-    return fn(q_rot, k_all, v_all, mask, scale), q_rot
+    out = fn(q_rot, k_all, v_all, mask, scale)
+    if gates is not None:
+        out = gate_output(out, gates if reference_dtype_flow else gates.float())
+    return out, q_rot
 
 
 # --------------------------------------------------------------------------------------

@@ -167,6 +167,40 @@ def test_fused_neighbours_match_torch_ops(gpu_device, dtype):
         assert_attn_close(out_f, out_u.float().cpu(), f"gated output t={t}")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_fused_neighbours_match_the_oracle(gpu_device, dtype):
+    """The one-call entry point with qk RMS norm, value-residual lerp and head gate inside the
+    kernels against the CPU oracle's layer_step with the same steps switched on
+    (src/model/attn.py:105-119): cache rows and RoPE(norm(q)) within 1 ulp of their row's largest
+    value (the kernel's row reduction order, rsqrt and the lerp's fused multiply-add differ in the
+    last bit), `written` identical, the gated output within 2e-2 / 2e-3 of the fp32 flow."""
+    dev = gpu_device
+    B, H, Hkv, T, Dh, n = 2, 4, 2, 128, 128, 3
+    p = Pair(dev, dtype, B=B, H=H, Hkv=Hkv, T=T, Dh=Dh, n_slots=n, cfg_id=62)
+    eps = torch.finfo(torch.float32).eps
+    g = torch.Generator("cpu").manual_seed(8)
+    lamb = torch.tensor(0.37, dtype=dtype)
+    layer = p.hip.layers[0]
+    for t in range(8):
+        frozen = t % 3 == 1
+        p.set_frozen(frozen)
+        q, k, v, pos = p.inputs(t)
+        q, k = q * 3, k * 0.5                                   # rows that are not already normalised
+        v1 = torch.randn(v.shape, generator=g).to(dtype)
+        gates = torch.sigmoid(torch.randn(B, T, H, generator=g)).to(dtype)          # [B, T, H] as the module has them
+        ref, q_rot = ro.layer_step(p.oracle, 0, q, k, v, pos, p.cos, p.sin, p.Hgrid, p.W, reference_dtype_flow=False,
+                                   qk_norm=True, v1=v1, v_lamb=lamb, gates=gates)
+        qd, kd, vd = merged_views(q.to(dev), k.to(dev), v.to(dev))
+        out, qrot_h = ops.rope_kv_attn(qd, kd, vd, to_dev(pos, dev), p.rope.cos, p.rope.sin, p.rope.height, p.rope.width,
+                                       layer.kv, layer.written, layer.L, 1, frozen, qk_norm_eps=eps, v1=v1.to(dev),
+                                       v_lamb=lamb.to(dev), gate=gates.to(dev).permute(0, 2, 1))
+        frac_q = _ulp_close(qrot_h, q_rot, f"RoPE(norm(q)) t={t}")
+        frac_kv = _ulp_close(layer.kv, p.oracle.layers[0].kv, f"cache t={t}")
+        assert frac_q < 0.02 and frac_kv < 0.02, (frac_q, frac_kv)
+        assert torch.equal(layer.written.cpu(), p.oracle.layers[0].written)
+        assert_attn_close(out, ref, f"gated output t={t}")
+
+
 def test_module_with_fused_neighbours(gpu_device):
     """RingAttn(fuse_elementwise=True) against the same module with the torch operations."""
     import types

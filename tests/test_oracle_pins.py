@@ -339,3 +339,96 @@ def test_synth_inputs_are_reproducible():
     assert all(torch.equal(x, y) for x, y in zip(a, b)) and not torch.equal(a[0], c[0])
     pos = ro.synth_pos_ids(9, 2, 16, 4)
     assert pos["t_pos"].unique().tolist() == [9] and pos["y_pos"][0].tolist() == [i // 4 for i in range(16)]
+
+
+# ------------------------------------------------------------------------------------------
+# the module's element-wise steps around the path (src/model/attn.py:105-109,117-119)
+# ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_rms_norm_matches_torch_and_closed_cases(dtype):
+    """The oracle's weightless RMS norm against F.rms_norm - the call the reference makes
+    (src/model/nn.py:55-56) - bit for bit, and against what the formula fixes."""
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(2, 3, 17, 128, generator=g) * 3).to(dtype)
+    got = ro.rms_norm(x)
+    assert got.dtype == dtype and torch.equal(got, F.rms_norm(x, (128,)))
+    # rows come out with unit root-mean-square (up to the rounding of the element type)
+    rms = got.float().pow(2).mean(-1).sqrt()
+    assert (rms - 1).abs().max().item() < {torch.bfloat16: 4e-3, torch.float16: 5e-4, torch.float32: 1e-6}[dtype]
+    # without the epsilon, scaling a row by a power of two changes nothing at all; with it, nothing
+    # beyond the last bit of a few elements (the epsilon is 1e-7 of a mean square near 9)
+    base0 = ro.rms_norm(x, eps=0.0)
+    assert torch.equal(ro.rms_norm(x * 4, eps=0.0), base0) and torch.equal(ro.rms_norm(x * 16, eps=0.0), base0)
+    assert (ro.rms_norm(x * 4) != got).float().mean().item() < 0.01
+    # a row of equal magnitudes normalises to +-1 exactly
+    c = torch.full((1, 1, 1, 64), 3.0).to(dtype)
+    c[..., ::2] = -3.0
+    out = ro.rms_norm(c)
+    assert torch.equal(out.abs(), torch.ones_like(out)) and torch.equal(out.sign(), c.sign())
+    # an all-zero row stays zero (eps keeps the reciprocal root finite)
+    assert torch.equal(ro.rms_norm(torch.zeros(1, 4, dtype=dtype)), torch.zeros(1, 4, dtype=dtype))
+    # a dropped mean (sum instead of mean) or a missing square root would not survive this
+    one = torch.zeros(1, 16, dtype=dtype)
+    one[0, 5] = 2.0
+    assert abs(ro.rms_norm(one)[0, 5].item() - 4.0) < 1e-5     # 2 / sqrt(4 / 16 + eps)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_value_lerp_matches_torch_and_end_points(dtype):
+    g = torch.Generator().manual_seed(4)
+    v = torch.randn(2, 3, 33, 64, generator=g).to(dtype)
+    v1 = torch.randn(2, 3, 33, 64, generator=g).to(dtype)
+    for w in (0.0, 0.25, 0.37, 0.5, 0.62, 1.0):
+        wt = torch.tensor(w, dtype=dtype)
+        got, want = ro.value_lerp(v, v1, wt), torch.lerp(v, v1, wt)
+        if dtype == torch.float32:      # torch contracts a + w*d into a fused multiply-add in fp32
+            assert (got - want).abs().max().item() <= 2.4e-7 * max(1.0, want.abs().max().item())
+        else:
+            assert torch.equal(got, want), f"w={w}"
+    assert torch.equal(ro.value_lerp(v, v1, torch.tensor(0.0, dtype=dtype)), v)
+    assert torch.equal(ro.value_lerp(v, v1, torch.tensor(1.0, dtype=dtype)), v1)
+    assert torch.equal(ro.value_lerp(v, v, torch.tensor(0.37, dtype=dtype)), v)
+    # direction: the weight moves the result towards v1, not away from it
+    a, b = torch.tensor([1.0], dtype=dtype), torch.tensor([3.0], dtype=dtype)
+    assert ro.value_lerp(a, b, torch.tensor(0.25, dtype=dtype)).item() == 1.5
+
+
+def test_gate_output_layout_and_rounding():
+    g = torch.Generator().manual_seed(5)
+    y = torch.randn(2, 4, 8, 16, generator=g).to(torch.bfloat16)          # [B, H, T, Dh]
+    gates = torch.rand(2, 8, 4, generator=g).to(torch.bfloat16)           # [B, T, H]
+    got = ro.gate_output(y, gates)
+    for b in range(2):
+        for h in range(4):
+            for t in range(8):
+                want = (y[b, h, t].float() * gates[b, t, h].float()).to(torch.bfloat16)
+                assert torch.equal(got[b, h, t], want)
+    assert torch.equal(ro.gate_output(y, torch.ones(2, 8, 4, dtype=torch.bfloat16)), y)
+    assert not ro.gate_output(y, torch.zeros(2, 8, 4, dtype=torch.bfloat16)).any()
+
+
+def test_layer_step_with_module_steps_equals_their_composition():
+    """layer_step with norm / lerp / gate switched on is exactly: torch's own lerp and rms_norm in
+    front of, and the tensor multiply behind, the plain layer_step (src/model/attn.py:105-119)."""
+    import torch.nn.functional as F
+    from types import SimpleNamespace
+    B, H, Hkv, T, Dh, n = 1, 4, 2, 16, 32, 2
+    cfg = SimpleNamespace(tokens_per_frame=T, local_window=n, global_window=n, global_attn_period=1,
+                          global_pinned_dilation=1, n_layers=1, n_heads=H, n_kv_heads=Hkv, d_model=H * Dh)
+    a, b = ro.OracleStaticKVCache(cfg, B, torch.bfloat16), ro.OracleStaticKVCache(cfg, B, torch.bfloat16)
+    a.set_frozen(False), b.set_frozen(False)
+    cos, sin = ro.rope_table_1d(8 * T, Dh)
+    g = torch.Generator().manual_seed(6)
+    lamb = torch.tensor(0.3, dtype=torch.bfloat16)
+    for t in range(4):
+        q, k, v = ro.synth_qkv(7, t, 0, B, H, Hkv, T, Dh, torch.bfloat16)
+        v1 = torch.randn(v.shape, generator=g).to(torch.bfloat16)
+        gates = torch.sigmoid(torch.randn(B, T, H, generator=g)).to(torch.bfloat16)
+        pos = ro.synth_pos_ids(t, B, T, 4)
+        out_a, qa = ro.layer_step(a, 0, q, k, v, pos, cos, sin, 4, 4, qk_norm=True, v1=v1, v_lamb=lamb, gates=gates)
+        out_b, qb = ro.layer_step(b, 0, F.rms_norm(q, (Dh,)), F.rms_norm(k, (Dh,)), torch.lerp(v, v1, lamb), pos,
+                                  cos, sin, 4, 4)
+        out_b = out_b * gates.permute(0, 2, 1).unsqueeze(-1)
+        assert torch.equal(qa, qb) and torch.equal(out_a, out_b)
+        assert torch.equal(a.layers[0].kv, b.layers[0].kv) and torch.equal(a.layers[0].written, b.layers[0].written)

@@ -26,7 +26,14 @@ class RoPE(nn.Module):
     """Table-driven rotary embedding (``src/model/attn.py:12-40``).  ``cos``/``sin`` are fp32
     ``[n_frames*height*width, Dh/2]`` buffers that ignore dtype casts of the parent model (the
     reference keeps them fp32 through ``NoCastModule``); the row of token ``(t, y, x)`` is
-    ``t*height*width + y*width + x``."""
+    ``t*height*width + y*width + x``.
+
+    As in the reference (``src/model/nn.py:10-24``), a dtype cast of a parent module leaves the
+    buffers fp32 but their *values* pass through the requested type: after ``model.to(bfloat16)``
+    the tables hold cos / sin rounded to bf16 precision.  This is what the reference's own tables
+    hold once ``WorldEngine`` has cast the model (``src/world_engine.py:56``), so it is kept; code
+    that wants full-precision angles must build the module after the cast, or move it with
+    ``.to(device)`` only."""
 
     def __init__(self, cos: Tensor, sin: Tensor, height: int, width: int):
         super().__init__()
