@@ -28,12 +28,6 @@ struct Bf16Mma {
     const bf16x2_t v = {f[2 * pair], f[2 * pair + 1]};
     return __builtin_amdgcn_fdot2_f32_bf16(v, ones, acc, false);
   }
-  // smallest bf16-representable value >= x (x finite)
-  __device__ static __forceinline__ float round_up(float x) {
-    uint32_t u = __float_as_uint(x);
-    u = (x >= 0.f) ? (u + 0xffffu) & 0xffff0000u : (u & 0xffff0000u);
-    return __uint_as_float(u);
-  }
 };
 struct F16Mma {
   typedef f16x8_t frag_t;
@@ -52,17 +46,6 @@ struct F16Mma {
     const f16x2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
     const f16x2_t v = {f[2 * pair], f[2 * pair + 1]};
     return __builtin_amdgcn_fdot2(v, ones, acc, false);
-  }
-  // smallest f16-representable value >= x (|x| well inside the f16 range)
-  __device__ static __forceinline__ float round_up(float x) {
-    const _Float16 h = (_Float16)x;  // nearest
-    float r = (float)h;
-    if (r < x) {
-      uint16_t b = __builtin_bit_cast(uint16_t, h);
-      b = (r >= 0.f) ? (uint16_t)(b + 1) : (uint16_t)(b - 1);
-      r = (float)__builtin_bit_cast(_Float16, b);
-    }
-    return r;
   }
 };
 

@@ -22,9 +22,10 @@
 // (lane i always lands at LDS offset 16*i) and undone in the fragment addresses.
 // Per 32-key block and wavefront:
 //   S^T = K Q^T        v_mfma_f32_32x32x16, A = K rows (ds_read_b128), B = Q in registers,
-//                      pre-multiplied by scale*log2(e); one extra MFMA (ones x -m_ref) makes the
-//                      logits leave the matrix core already shifted by the running reference.
-//   P = 2^S            v_exp_f32 + v_cvt_pk + v_dot2c row sum; each lane owns one query column.
+//                      multiplied by a power of two (exact).
+//   P = 2^((S-m) c)    one fused multiply-add per logit applies the rest of the softmax scale
+//                      (c in [1, 2)) and the running reference m, then v_exp_f32 + v_cvt_pk +
+//                      v_dot2c row sum; each lane owns one query column.
 //   O^T += V^T P^T     A = V^T via ds_read_b64_tr_b16, B = P straight from registers.
 // The three are software-pipelined across blocks (logits of block i+1 and product of block i-1
 // run on the matrix cores while the VALU handles block i); LDS fragment reads are stated up to 15
@@ -47,10 +48,6 @@
 #include "../../include/we_attn.h"
 
 #include <atomic>
-
-#ifndef WE_SHIFT_IN_ACC
-#define WE_SHIFT_IN_ACC 0
-#endif
 
 namespace we {
 
@@ -304,33 +301,16 @@ attn_ring_kernel(AttnParams p) {
   float m_ref = -INFINITY, l_run = 0.f;
 
   const f32x16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  // The logits leave the matrix core already shifted by the running reference exponent of this
-  // lane's query (every lane owns one query column of the transposed scores), in one of two ways:
-  //  * WE_SHIFT_IN_ACC: the first product of a block accumulates onto a register block that holds
-  //    -m_ref in all 16 elements; no instruction per block, 16 registers.
-  //  * otherwise: one extra MFMA per block, ones (K side, contraction index 0) x -m_ref (Q side);
-  //    m_ref is kept representable in the element type for that.  8 registers.
-#if WE_SHIFT_IN_ACC
-  f32x16_t shiftv = zero16;
-  auto set_shift = [&]() __attribute__((always_inline)) {
-#pragma unroll
-    for (int i = 0; i < 16; ++i) shiftv[i] = -m_ref;
-  };
-#else
-  frag_t ones_frag = __builtin_bit_cast(frag_t, u32x4_t{0u, 0u, 0u, 0u});
-  if (hh == 0) ones_frag[0] = (typename M::elem_t)1.0f;
-  frag_t shift = __builtin_bit_cast(frag_t, u32x4_t{0u, 0u, 0u, 0u});
-  auto set_shift = [&]() __attribute__((always_inline)) {
-    shift = __builtin_bit_cast(frag_t, u32x4_t{0u, 0u, 0u, 0u});
-    if (hh == 0) shift[0] = (typename M::elem_t)(-m_ref);
-  };
-#endif
-  // Softmax scale: q is multiplied by an exact power of two (no rounding of the element-type
-  // values, so the logits are the exact products' sums), the remaining factor in [1, 2) is
-  // applied to the shifted logits in fp32 inside the exponentials.
+  // Softmax scale and reference: q is multiplied by an exact power of two (no rounding of the
+  // element-type values, so the logits are the exact products' sums); the remaining factor lmul in
+  // [1, 2) and the running reference m_ref of this lane's query (every lane owns one query column
+  // of the transposed scores) are applied by one fused multiply-add per logit in front of its
+  // exponential: p = 2^(s * lmul + msc), msc = -m_ref * lmul.
   const float lmul = p.logit_mul;
+  float msc = 0.f;
+  auto set_shift = [&]() __attribute__((always_inline)) { msc = -m_ref * lmul; };
 
-  // probabilities of one 32-key block from its shifted logits: p = 2^(s - sub), packed to the
+  // probabilities of one 32-key block from its logits: p = 2^((s - sub) * lmul), packed to the
   // element type; returns this half-wave's share of the row sum (of the rounded values)
   auto probabilities = [&](frag_t(&pf)[2], const f32x16_t& s, float sub) __attribute__((always_inline)) {
     float rs = 0.f;
@@ -355,7 +335,7 @@ attn_ring_kernel(AttnParams p) {
   };
 
   // The pipeline runs on 32-key blocks.  One step computes, for this wavefront,
-  //   matrix cores: the shifted logits of the block read at K offset KOFF (-> s_next) and the
+  //   matrix cores: the logits of the block read at K offset KOFF (-> s_next) and the
   //                 product of the previous block's probabilities with the V block at VOFF;
   //   VALU:         the probabilities of the current block (s_cur -> p_cur).
   // LDS reads are issued in consumption order - K fragments 0..KS-1, then the NV V^T fragments
@@ -426,34 +406,22 @@ attn_ring_kernel(AttnParams p) {
 #pragma unroll
       for (int t = 0; t < EPS; ++t)
         if (g * EPS + t < 16) {
-          e[g * EPS + t] = __builtin_amdgcn_exp2f(s_cur[g * EPS + t] * lmul);
+          e[g * EPS + t] = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[g * EPS + t], lmul, msc));
           // an exponential has no side effect, so nothing else keeps it in its slot: left alone the
           // compiler sinks the first nine of a step below the tile DMAs
           asm volatile("" : "+v"(e[g * EPS + t]));
         }
     };
-#if WE_SHIFT_IN_ACC
-    constexpr int S0 = 0;   // slot of the exponentials that follow the first logits product
     f32x16_t s_next;
-#else
-    constexpr int S0 = 1;   // slot 0 follows the shift product
-    f32x16_t s_next = M::mma(ones_frag, shift, zero16);
-    exp_slot(0);
-    __builtin_amdgcn_sched_barrier(0);
-#endif
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-#if WE_SHIFT_IN_ACC
-      s_next = M::mma(__builtin_bit_cast(frag_t, kf[ks]), qf[ks], ks == 0 ? shiftv : s_next);
-#else
-      s_next = M::mma(__builtin_bit_cast(frag_t, kf[ks]), qf[ks], s_next);
-#endif
+      s_next = M::mma(__builtin_bit_cast(frag_t, kf[ks]), qf[ks], ks == 0 ? zero16 : s_next);
       // keep the read queue full without exceeding the 15 reads the counter can track
       if (vnext < NV && ks <= 12 - KS) {
         read_v(voff_c, vnext);
         ++vnext;
         }
-      exp_slot(S0 + ks);
+      exp_slot(ks);
       __builtin_amdgcn_sched_barrier(0);
     }
     mid();  // the tile DMAs of this iteration go out here, under the MFMAs already queued
@@ -469,7 +437,7 @@ attn_ring_kernel(AttnParams p) {
       o[i % DB] = M::mma(__builtin_bit_cast(frag_t, a4), p_prev[i / DB], o[i % DB]);
       if (i >= I0 && npair < NPAIR) next_pair();
       // VALU slices: the last exponentials; packing of the two 16-key halves and their row sums
-      exp_slot(S0 + KS + i);
+      exp_slot(KS + i);
       if (i == 1) p_cur[0] = M::pack8(e[0], e[1], e[2], e[3], e[4], e[5], e[6], e[7]);
       if (i == 2) {
 #pragma unroll
@@ -487,20 +455,16 @@ attn_ring_kernel(AttnParams p) {
     const bool seed = RAGGED && ref_unset && cur_keys > 0;
     if (seed || __ballot(!(rs <= 256.f)) != 0ull) {
       // Rare: some probability of this block may exceed 2^8.  Raise the reference of the rows
-      // that need it, redo the block's probabilities exactly, re-base the logits of the next
-      // block, which were produced with the old reference, and rescale the accumulators: they hold
-      // the blocks before this one (the last of those products was issued above).
+      // that need it, redo the block's probabilities exactly and rescale the accumulators: they
+      // hold the blocks before this one (the last of those products was issued above).
       const float mx = block_max(s_cur);
-      const float m_new = (seed ? mx > -INFINITY : mx > 0.f) ? M::round_up(m_ref + mx) : m_ref;
-      const float delta = m_new - m_ref;
-      const float alpha = seed ? 1.f : __builtin_amdgcn_exp2f(-delta * lmul);  // seed: sums and accumulators are still zero
+      const float m_new = (seed ? mx > -INFINITY : mx > m_ref) ? mx : m_ref;
+      const float alpha = seed ? 1.f : __builtin_amdgcn_exp2f((m_ref - m_new) * lmul);  // seed: sums and accumulators are still zero
       if (RAGGED) ref_unset = false;
-      rs = probabilities(p_cur, s_cur, delta);
+      rs = probabilities(p_cur, s_cur, m_new);
       l_run *= alpha;
       m_ref = m_new;
       set_shift();
-#pragma unroll
-      for (int i = 0; i < 16; ++i) s_next[i] -= delta;
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -563,7 +527,7 @@ attn_ring_kernel(AttnParams p) {
     }
     dma_wait<(KA + 1) * NDMA>();
     __syncthreads();  // K(0) and the zeroed V slot are in LDS
-    // first block: plain logits, reference = its row max, shifted by hand
+    // first block: reference = its row max
     {
       s_cur = zero16;
 #pragma unroll
@@ -574,14 +538,12 @@ attn_ring_kernel(AttnParams p) {
       const int nk0 = block_keys(csub, hb);
       if (RAGGED && nk0 < 32) mask_keys(s_cur, nk0);
       const float mx0 = block_max(s_cur);
-      m_ref = mx0 > -INFINITY ? M::round_up(mx0) : 0.f;  // (a block of the first tile may be empty)
+      m_ref = mx0 > -INFINITY ? mx0 : 0.f;  // (a block of the first tile may be empty)
       if (RAGGED) {
         ref_unset = nk0 == 0;
         cur_keys = nk0;
       }
       set_shift();
-#pragma unroll
-      for (int i = 0; i < 16; ++i) s_cur[i] -= m_ref;
     }
     dma_wait<2 * NDMA>();
     __syncthreads();  // everything but the last K and V tile issued so far has landed
