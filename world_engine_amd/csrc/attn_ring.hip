@@ -21,10 +21,10 @@
 // conflicts are avoided by XOR-swizzling 16-byte chunks, applied on the global side of the DMA
 // (lane i always lands at LDS offset 16*i) and undone in the fragment addresses.
 // Per 32-key block and wavefront:
-//   S^T = K Q^T        v_mfma_f32_32x32x16, A = K rows (ds_read_b128), B = Q in registers,
-//                      multiplied by a power of two (exact).
-//   P = 2^((S-m) c)    one fused multiply-add per logit applies the rest of the softmax scale
-//                      (c in [1, 2)) and the running reference m, then v_exp_f32 + v_cvt_pk +
+//   S^T = K Q^T        v_mfma_f32_32x32x16, A = K rows (ds_read_b128), B = Q in registers as
+//                      loaded (no scaling, so nothing is rounded in front of the matrix core).
+//   P = 2^((S-m) c)    one fused multiply-add per logit applies the softmax scale (c = scale *
+//                      log2 e) and the running reference m, then v_exp_f32 + v_cvt_pk +
 //                      v_dot2c row sum; each lane owns one query column.
 //   O^T += V^T P^T     A = V^T via ds_read_b64_tr_b16, B = P straight from registers.
 // The three are software-pipelined across blocks (logits of block i+1 and product of block i-1
@@ -301,12 +301,12 @@ attn_ring_kernel(AttnParams p) {
   float m_ref = -INFINITY, l_run = 0.f;
 
   const f32x16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  // Softmax scale and reference: q is multiplied by an exact power of two (no rounding of the
-  // element-type values, so the logits are the exact products' sums); the remaining factor lmul in
-  // [1, 2) and the running reference m_ref of this lane's query (every lane owns one query column
-  // of the transposed scores) are applied by one fused multiply-add per logit in front of its
-  // exponential: p = 2^(s * lmul + msc), msc = -m_ref * lmul.
-  const float lmul = p.logit_mul;
+  // Softmax scale and reference: the logits are the exact products' sums of the element-type q
+  // and k (nothing is rounded before the matrix core); the scale c = softmax scale * log2(e) and
+  // the running reference m_ref of this lane's query (every lane owns one query column of the
+  // transposed scores) are applied by one fused multiply-add per logit in front of its
+  // exponential: p = 2^(s * c + msc), msc = -m_ref * c.
+  const float lmul = p.scale_log2;
   float msc = 0.f;
   auto set_shift = [&]() __attribute__((always_inline)) { msc = -m_ref * lmul; };
 
@@ -516,15 +516,7 @@ attn_ring_kernel(AttnParams p) {
       }
       dma_v(o1, 1);
     }
-    // ---- Q stays in registers for the whole kernel, multiplied by a power of two (exact); done
-    //      while the first tiles are on their way ----
-    const float c2 = p.q_pow2;
-  #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const frag_t raw = qf[ks];
-      qf[ks] = M::pack8((float)raw[0] * c2, (float)raw[1] * c2, (float)raw[2] * c2, (float)raw[3] * c2,
-                        (float)raw[4] * c2, (float)raw[5] * c2, (float)raw[6] * c2, (float)raw[7] * c2);
-    }
+    // (Q stays in registers for the whole kernel, as loaded)
     dma_wait<(KA + 1) * NDMA>();
     __syncthreads();  // K(0) and the zeroed V slot are in LDS
     // first block: reference = its row max
@@ -623,7 +615,7 @@ attn_ring_kernel(AttnParams p) {
   float lo, up;
   half_wave_pair(l_run, lo, up);
   float l_tot = lo + up;
-  m_ref *= lmul;  // from the matrix core's units (logits / lmul) to the log2 domain the merges work in
+  m_ref *= lmul;  // from raw logits to the log2 domain the merges work in
 
   if (KSPLIT == 2) {
     // ---- the two wavefronts of a query block merge their (m, l, O) through LDS ----

@@ -55,8 +55,8 @@ __global__ void __launch_bounds__(256) attn_ring_f32_kernel(AttnParams p) {
 #pragma unroll
     for (int d = 0; d < PART; d += 4) {
       const f32x4_t x = *reinterpret_cast<const f32x4_t*>(src + d);
-      q[d] = x[0] * (p.q_pow2 * p.logit_mul); q[d + 1] = x[1] * (p.q_pow2 * p.logit_mul);
-      q[d + 2] = x[2] * (p.q_pow2 * p.logit_mul); q[d + 3] = x[3] * (p.q_pow2 * p.logit_mul);
+      q[d] = x[0] * p.scale_log2; q[d + 1] = x[1] * p.scale_log2;
+      q[d + 2] = x[2] * p.scale_log2; q[d + 3] = x[3] * p.scale_log2;
     }
   }
   float o[PART];

@@ -3,7 +3,6 @@
 #include "../../include/we_attn.h"
 #include "we_kernels.h"
 
-#include <cmath>
 #include <mutex>
 
 // Split-context partial results of we_attn_ring_fwd_static: part of the library's device image, so
@@ -194,13 +193,7 @@ int prepare_attn(const void* q, const int64_t* q_strides, const void* kv, const 
   p.group = H / Hkv;
   p.members = p.group * p.q_tiles;
   p.unit_splits = pl.units_whole + (B * Hkv - pl.units_whole) * pl.n_splits;
-  {
-    const float c2 = scale * 1.4426950408889634f;
-    int ex = 0;
-    const float mant = frexpf(c2, &ex);       // c2 = mant * 2^ex, mant in [0.5, 1)
-    p.q_pow2 = ldexpf(1.f, ex - 1);
-    p.logit_mul = mant * 2.f;
-  }
+  p.scale_log2 = scale * 1.4426950408889634f;
   p.gate = nullptr; p.gs_b = p.gs_h = p.gs_t = 0;
 
   if ((p.unit_splits + 7) / 8 > 65535 || p.group > 65535 || (int64_t)B * H - (int64_t)pl.units_whole * p.group > 65535)

@@ -55,9 +55,7 @@ struct AttnParams {
   int group;        // query heads per kv head, H / Hkv
   int members;      // workgroups that share one K/V stream: group * q_tiles
   int unit_splits;  // units_whole + (B * Hkv - units_whole) * n_splits
-  // softmax scale * log2(e) = q_pow2 * logit_mul: q is multiplied by q_pow2, a power of two (exact in
-  // the element type), the logits by logit_mul in [1, 2) in fp32
-  float q_pow2, logit_mul;
+  float scale_log2;  // softmax scale * log2(e), applied to the raw logits in fp32
   // optional per (batch, head, token) output gate, element type (src/model/attn.py:117-119)
   const void* gate;
   int64_t gs_b, gs_h, gs_t;
