@@ -108,6 +108,9 @@ def read_traffic(cfg_id):
     (profiles/attn_ring_cfgN_hbm_traffic.txt: two rocprofv3 --pmc runs, FETCH_SIZE and WRITE_SIZE,
     each scaled by the same counter's reading for a copy kernel of known size).  None when there is
     no summary."""
+    note = ""
+    if cfg_id == 2:      # 24 layers of cfg1 shapes: one attention call moves what a cfg1 call moves
+        cfg_id, note = 1, " (cfg2 = 24 layers of cfg1 shapes; per attention call)"
     path = os.path.join(ROOT, "profiles", f"attn_ring_cfg{cfg_id}_hbm_traffic.txt")
     try:
         text = open(path).read()
@@ -120,7 +123,7 @@ def read_traffic(cfg_id):
     rev = re.search(r"kernel sources at commit\s+([0-9a-f]{7,40})", text)
     if rev:
         src += f" (kernel sources at commit {rev.group(1)})"
-    return int(m.group(1)), src
+    return int(m.group(1)), src + note
 
 
 def cfg_namespace(c, layers):
@@ -300,6 +303,31 @@ def run_gpu(cfg_id, c, args, torch, ro, wea, ops):
                  "algorithmic_bytes": byts, "algorithmic_flops": flops, "n_splits": n_splits,
                  "tflops": round(tflops, 2), "algorithmic_gbps": round(gbps, 1)})
     log(f"[bench] attention call: {attn_us:.2f} us -> {tflops:.1f} TFLOP/s, {gbps:.0f} GB/s algorithmic")
+
+    # ---- shader clock inside the main kernel: cycles against the constant 100 MHz counter, per workgroup ----
+    if not args.eager:
+        try:
+            clocks = torch.zeros(2 * 65536, dtype=torch.int64, device=dev)
+            for _ in range(60):                       # back to back, so the board sits at its sustained clock
+                ops.attn_ring(q_rot, layer0.kv, layer0.written, pos["t_pos"], layer0.L, 1, n_splits=args.n_splits,
+                              q_tile=args.q_tile, out=out, workspace=ws, clocks=clocks)
+            torch.cuda.synchronize()
+            ck = clocks.view(-1, 2).cpu()
+            ck = ck[ck[:, 1] > 0].double()
+            ghz = (ck[:, 0] / (ck[:, 1] * 10.0)).tolist()          # cycles per 10 ns tick
+            wg_us = (ck[:, 1] / 100.0).tolist()
+            roof["shader_clock"] = {"ghz_median": round(percentile(ghz, 0.5), 3), "ghz_p10": round(percentile(ghz, 0.1), 3),
+                                    "ghz_p90": round(percentile(ghz, 0.9), 3), "workgroups": len(ghz),
+                                    "workgroup_us_median": round(percentile(wg_us, 0.5), 2),
+                                    "workgroup_us_max": round(max(wg_us), 2),
+                                    "what": "attn_ring_kernel, 60 launches back to back, last launch: cycles of the shader "
+                                            "clock per workgroup over the same interval on the constant 100 MHz counter"}
+            log(f"[bench] shader clock inside attn_ring_kernel: {roof['shader_clock']['ghz_median']} GHz "
+                f"(workgroups run {roof['shader_clock']['workgroup_us_median']} us, longest {roof['shader_clock']['workgroup_us_max']} us)")
+            del clocks
+        except Exception as e:                      # noqa: BLE001 - a missing figure, not a failed benchmark
+            roof["shader_clock"] = None
+            log(f"[bench] shader clock not measured: {e!r}")
     res = {"workload": c["name"], "us_per_step": round(st["median"], 3), "us_per_step_p10": round(st["p10"], 3),
            "us_per_step_p90": round(st["p90"], 3), "samples": st["samples"], "replays_per_sample": reps,
            "us_per_layer_step": round(st["median"] / layers, 3), "layers": layers, "calls_per_frame": subs,
@@ -441,6 +469,9 @@ def main():
     ap.add_argument("--eager", action="store_true", help="launch from Python per call instead of a HIP graph")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-module", action="store_true", help="skip the module-level timing")
+    ap.add_argument("--module-only", action="store_true",
+                    help="only the module-level timing (RingAttn.forward at cfg1 shapes, torch and fused element-wise "
+                         "neighbours): what a kernel trace of the module is taken from")
     ap.add_argument("--no-peaks", action="store_true", help="skip the measured GEMM / copy rates of this box")
     ap.add_argument("--two-calls", action="store_true",
                     help="we_rope_kv_store + we_attn_ring_fwd instead of the one-call we_rope_kv_attn_fwd")
@@ -465,6 +496,9 @@ def main():
     from world_engine_amd import ops
 
     torch.cuda.set_device(0)
+    if args.module_only:
+        print(json.dumps({"module": run_module(args, torch, ro, wea)}), flush=True)
+        return
     single = args.config != 0
     cfg_ids = [args.config] if single else sorted(CONFIGS)
     head = args.config if single else HEADLINE

@@ -160,6 +160,24 @@ int we_attn_ring_fwd(const void* q, const int64_t q_strides[3],
                      int32_t dtype, void* stream);
 
 /*
+ * Measurement aid without a counterpart in the reference: we_attn_ring_fwd that also records how
+ * long every workgroup of the main kernel ran, on two clocks.  clocks[2 * w] receives workgroup
+ * w's duration in shader-clock cycles, clocks[2 * w + 1] the same interval in ticks of the
+ * device's constant 100 MHz counter, w being the linear workgroup id of the launch; their ratio
+ * is the shader clock the kernel actually ran at (boards lower it under their power limit).
+ * clocks_len = number of uint64 elements available; at least 2 * (workgroups of the launch) or
+ * WE_ERR_WORKSPACE is returned; entries of workgroups that own no work stay untouched (zero them
+ * beforehand).  bf16 / f16 only.  Everything else as we_attn_ring_fwd.
+ */
+int we_attn_ring_fwd_clocked(const void* q, const int64_t q_strides[3],
+                             const void* kv, const uint8_t* written, const int64_t* t_pos,
+                             void* out, const int64_t out_strides[3],
+                             void* workspace, size_t workspace_bytes,
+                             int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L,
+                             int32_t dilation, float scale, int32_t n_splits, int32_t q_tile,
+                             int32_t dtype, uint64_t* clocks, size_t clocks_len, void* stream);
+
+/*
  * we_attn_ring_fwd for callers that cannot allocate device memory, not even a workspace: code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
  * counterpart in the reference (whose attention call allocates through torch as it pleases).

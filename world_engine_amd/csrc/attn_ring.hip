@@ -136,6 +136,9 @@ attn_ring_kernel(AttnParams p) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, hh = lane >> 5;
+  // measurement aid: shader-clock and constant-rate (100 MHz) counters at the workgroup's start
+  const uint64_t clk0 = p.clock_out != nullptr ? (uint64_t)__builtin_readcyclecounter() : 0;
+  const uint64_t wall0 = p.clock_out != nullptr ? (uint64_t)__builtin_amdgcn_s_memrealtime() : 0;
   const int qb = wave % QW;   // query block of this wavefront
   const int hb = wave / QW;   // key block of every tile it handles when KSPLIT == 2 (else 0)
 
@@ -710,6 +713,11 @@ attn_ring_kernel(AttnParams p) {
         }
       }
     }
+  }
+  if (p.clock_out != nullptr && tid == 0) {
+    const uint64_t wg = blockIdx.x + (uint64_t)gridDim.x * (blockIdx.y + (uint64_t)gridDim.y * blockIdx.z);
+    p.clock_out[2 * wg] = (uint64_t)__builtin_readcyclecounter() - clk0;
+    p.clock_out[2 * wg + 1] = (uint64_t)__builtin_amdgcn_s_memrealtime() - wall0;
   }
 }
 

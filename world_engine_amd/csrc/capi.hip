@@ -195,6 +195,7 @@ int prepare_attn(const void* q, const int64_t* q_strides, const void* kv, const 
   p.unit_splits = pl.units_whole + (B * Hkv - pl.units_whole) * pl.n_splits;
   p.scale_log2 = scale * 1.4426950408889634f;
   p.gate = nullptr; p.gs_b = p.gs_h = p.gs_t = 0;
+  p.clock_out = nullptr;
 
   if ((p.unit_splits + 7) / 8 > 65535 || p.group > 65535 || (int64_t)B * H - (int64_t)pl.units_whole * p.group > 65535)
     return WE_ERR_UNSUPPORTED;  // grid y / z limits of the two launches
@@ -304,6 +305,24 @@ int we_attn_ring_fwd(const void* q, const int64_t q_strides[3], const void* kv, 
   if (rc != WE_OK) return rc;
   hipStream_t st = static_cast<hipStream_t>(stream);
   return launch_attn(p, pl, Dh, dtype, st);
+}
+
+int we_attn_ring_fwd_clocked(const void* q, const int64_t q_strides[3], const void* kv, const uint8_t* written,
+                             const int64_t* t_pos, void* out, const int64_t out_strides[3], void* workspace,
+                             size_t workspace_bytes, int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh,
+                             int64_t L, int32_t dilation, float scale, int32_t n_splits, int32_t q_tile,
+                             int32_t dtype, uint64_t* clocks, size_t clocks_len, void* stream) {
+  if (!clocks) return WE_ERR_NULL_POINTER;
+  if (dtype == WE_DTYPE_F32) return WE_ERR_UNSUPPORTED;
+  we::AttnParams p;
+  AttnPlan pl;
+  const int rc = prepare_attn(q, q_strides, kv, written, t_pos, out, out_strides, workspace, workspace_bytes, B, H,
+                              Hkv, T, Dh, L, dilation, scale, n_splits, q_tile, dtype, p, pl);
+  if (rc != WE_OK) return rc;
+  const size_t wgs = (size_t)(8 * p.q_tiles) * (size_t)p.group * (size_t)((p.unit_splits + 7) / 8);
+  if (clocks_len < 2 * wgs) return WE_ERR_WORKSPACE;
+  p.clock_out = clocks;
+  return launch_attn(p, pl, Dh, dtype, static_cast<hipStream_t>(stream));
 }
 
 int we_attn_ring_fwd_static(const void* q, const int64_t q_strides[3], const void* kv, const uint8_t* written,

@@ -59,6 +59,9 @@ struct AttnParams {
   // optional per (batch, head, token) output gate, element type (src/model/attn.py:117-119)
   const void* gate;
   int64_t gs_b, gs_h, gs_t;
+  // measurement aid (null = off): every workgroup of the main kernel leaves its duration as
+  // (shader-clock cycles, ticks of the constant 100 MHz counter) at [2 * linear workgroup id]
+  uint64_t* clock_out;
 };
 
 hipError_t launch_rope_kv_store(const StoreParams& p, int dtype, hipStream_t stream);

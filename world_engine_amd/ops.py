@@ -163,7 +163,7 @@ def attn_workspace_bytes(B: int, H: int, Hkv: int, T: int, Dh: int, L: int, n_sp
 def attn_ring(q: Tensor, kv: Tensor, written: Tensor, t_pos: Tensor, L: int, dilation: int,
               scale: Optional[float] = None, n_splits: int = 0, q_tile: int = 0,
               out: Optional[Tensor] = None, workspace: Optional[Tensor] = None,
-              token_major_out: bool = True) -> Tensor:
+              token_major_out: bool = True, clocks: Optional[Tensor] = None) -> Tensor:
     """Attention of one frame's queries over the visible part of the ring buffer.
 
     Replaces ``make_block_mask`` + ``flex_attention`` (``src/model/kv_cache.py:141-144``,
@@ -171,6 +171,8 @@ def attn_ring(q: Tensor, kv: Tensor, written: Tensor, t_pos: Tensor, L: int, dil
     ``[2,B,Hkv,L+T,Dh]``, ``written`` ``[L+T]`` bool, ``t_pos`` int64 with the frame index at
     element 0.  Returns ``[B,H,T,Dh]``; with ``token_major_out`` its memory is ``[B,T,H,Dh]`` so
     that ``y.transpose(1, 2).reshape(B, T, H*Dh)`` is a view (``src/patch_model.py:139``).
+    ``clocks`` (int64 device tensor, measurement aid): per workgroup of the main kernel its duration
+    in shader-clock cycles and in ticks of the constant 100 MHz counter (``we_attn_ring_fwd_clocked``).
     """
     dev = _need_device(q, kv, written, t_pos)
     if q.dim() != 4:
@@ -197,13 +199,19 @@ def attn_ring(q: Tensor, kv: Tensor, written: Tensor, t_pos: Tensor, L: int, dil
             out = torch.empty((B, H, T, Dh), dtype=q.dtype, device=dev)
     elif tuple(out.shape) != (B, H, T, Dh) or out.dtype != q.dtype or out.device != dev:
         raise RuntimeError("out must be [B, H, T, Dh] of q's element type on q's device")
-    code = lib.we_attn_ring_fwd(
-        q.data_ptr(), _bhtd_strides(q, "q"), kv.data_ptr(), written.data_ptr(), t_pos.data_ptr(),
-        out.data_ptr(), _bhtd_strides(out, "out"),
-        workspace.data_ptr() if ws_bytes else None,
-        workspace.numel() * workspace.element_size() if ws_bytes else 0,
-        B, H, Hkv, T, Dh, L, dilation, scale, n_splits, q_tile, _dtype_code(q), _stream_ptr(dev))
-    _capi.check(code, "we_attn_ring_fwd")
+    common = (q.data_ptr(), _bhtd_strides(q, "q"), kv.data_ptr(), written.data_ptr(), t_pos.data_ptr(),
+              out.data_ptr(), _bhtd_strides(out, "out"),
+              workspace.data_ptr() if ws_bytes else None,
+              workspace.numel() * workspace.element_size() if ws_bytes else 0,
+              B, H, Hkv, T, Dh, L, dilation, scale, n_splits, q_tile, _dtype_code(q))
+    if clocks is not None:
+        if clocks.dtype != torch.int64 or not clocks.is_contiguous() or clocks.device != dev:
+            raise RuntimeError("clocks must be a contiguous int64 tensor on q's device")
+        code = lib.we_attn_ring_fwd_clocked(*common, clocks.data_ptr(), clocks.numel(), _stream_ptr(dev))
+        _capi.check(code, "we_attn_ring_fwd_clocked")
+    else:
+        code = lib.we_attn_ring_fwd(*common, _stream_ptr(dev))
+        _capi.check(code, "we_attn_ring_fwd")
     return out
 
 
