@@ -215,8 +215,16 @@ int we_attn_ring_fwd_static(const void* q, const int64_t q_strides[3],
  *   gate         out[b, h, t, :] *= gate[b, h, t] (sigmoid already applied), element strides
  *                gate_strides = {batch, head, token}; the attention output is rounded to the
  *                element type first, as the module's own multiply sees it.  NULL = off.
- * Results equal the separate torch operations up to the last bit of the row reduction and of the
- * lerp's fused multiply-add (1 ulp of the element type); the gate multiply is exact.
+ *   gate_x, gate_w   instead of `gate`: the gate is computed in the kernels' epilogues as
+ *                sigmoid(gate_proj(x[..., :H])) (src/model/attn.py:117-118), which saves the module
+ *                a GEMM launch and a sigmoid launch per layer.  gate_x points at x[b, t, 0] of the
+ *                module's input [B, T, >= H] (channel stride 1, element strides gate_x_strides =
+ *                {batch, token}), gate_w at gate_proj.weight [H, H] row-major (out, in).  The
+ *                projection's output and the sigmoid's are rounded to the element type like the
+ *                module's tensors.  Both NULL = off; not together with `gate`; bf16 / f16 only.
+ * Results equal the separate torch operations up to the last bit of the row reduction, of the
+ * lerp's fused multiply-add and of the gate's dot product (1 ulp of the element type); the gate
+ * multiply itself is exact.
  */
 typedef struct we_attn_extras {
   float qk_norm_eps;
@@ -225,6 +233,9 @@ typedef struct we_attn_extras {
   const void* v_lamb;
   const void* gate;
   int64_t gate_strides[3];
+  const void* gate_x;
+  int64_t gate_x_strides[2];
+  const void* gate_w;
 } we_attn_extras;
 
 /*

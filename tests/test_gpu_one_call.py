@@ -167,13 +167,16 @@ def test_fused_neighbours_match_torch_ops(gpu_device, dtype):
         assert_attn_close(out_f, out_u.float().cpu(), f"gated output t={t}")
 
 
+@pytest.mark.parametrize("gate_mode", ["given", "projected"])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_fused_neighbours_match_the_oracle(gpu_device, dtype):
+def test_fused_neighbours_match_the_oracle(gpu_device, dtype, gate_mode):
     """The one-call entry point with qk RMS norm, value-residual lerp and head gate inside the
     kernels against the CPU oracle's layer_step with the same steps switched on
     (src/model/attn.py:105-119): cache rows and RoPE(norm(q)) within 1 ulp of their row's largest
     value (the kernel's row reduction order, rsqrt and the lerp's fused multiply-add differ in the
-    last bit), `written` identical, the gated output within 2e-2 / 2e-3 of the fp32 flow."""
+    last bit), `written` identical, the gated output within 2e-2 / 2e-3 of the fp32 flow.  The
+    gate is either handed over ready-made or projected from the module's input inside the kernels
+    (sigmoid(gate_proj(x[..., :H])), src/model/attn.py:117-118)."""
     dev = gpu_device
     B, H, Hkv, T, Dh, n = 2, 4, 2, 128, 128, 3
     p = Pair(dev, dtype, B=B, H=H, Hkv=Hkv, T=T, Dh=Dh, n_slots=n, cfg_id=62)
@@ -187,13 +190,20 @@ def test_fused_neighbours_match_the_oracle(gpu_device, dtype):
         q, k, v, pos = p.inputs(t)
         q, k = q * 3, k * 0.5                                   # rows that are not already normalised
         v1 = torch.randn(v.shape, generator=g).to(dtype)
-        gates = torch.sigmoid(torch.randn(B, T, H, generator=g)).to(dtype)          # [B, T, H] as the module has them
+        if gate_mode == "given":
+            gates = torch.sigmoid(torch.randn(B, T, H, generator=g)).to(dtype)      # [B, T, H] as the module has them
+            gate_kw = dict(gate=gates.to(dev).permute(0, 2, 1))
+        else:
+            x_full = (torch.randn(B, T, 3 * H, generator=g) * 2).to(dtype)          # the module's input; the gate reads its first H channels
+            w_gate = (torch.randn(H, H, generator=g) * 0.7).to(dtype)
+            gates = torch.sigmoid(torch.nn.functional.linear(x_full[..., :H], w_gate))
+            gate_kw = dict(gate_x=x_full.to(dev)[..., :H], gate_w=w_gate.to(dev))
         ref, q_rot = ro.layer_step(p.oracle, 0, q, k, v, pos, p.cos, p.sin, p.Hgrid, p.W, reference_dtype_flow=False,
                                    qk_norm=True, v1=v1, v_lamb=lamb, gates=gates)
         qd, kd, vd = merged_views(q.to(dev), k.to(dev), v.to(dev))
         out, qrot_h = ops.rope_kv_attn(qd, kd, vd, to_dev(pos, dev), p.rope.cos, p.rope.sin, p.rope.height, p.rope.width,
                                        layer.kv, layer.written, layer.L, 1, frozen, qk_norm_eps=eps, v1=v1.to(dev),
-                                       v_lamb=lamb.to(dev), gate=gates.to(dev).permute(0, 2, 1))
+                                       v_lamb=lamb.to(dev), **gate_kw)
         frac_q = _ulp_close(qrot_h, q_rot, f"RoPE(norm(q)) t={t}")
         frac_kv = _ulp_close(layer.kv, p.oracle.layers[0].kv, f"cache t={t}")
         assert frac_q < 0.02 and frac_kv < 0.02, (frac_q, frac_kv)

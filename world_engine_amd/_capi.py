@@ -22,7 +22,8 @@ _I64x3 = POINTER(c_int64)
 class AttnExtras(ctypes.Structure):
     """``we_attn_extras`` of include/we_attn.h."""
     _fields_ = [("qk_norm_eps", ctypes.c_float), ("v1", c_void_p), ("v1_strides", ctypes.c_int64 * 3),
-                ("v_lamb", c_void_p), ("gate", c_void_p), ("gate_strides", ctypes.c_int64 * 3)]
+                ("v_lamb", c_void_p), ("gate", c_void_p), ("gate_strides", ctypes.c_int64 * 3),
+                ("gate_x", c_void_p), ("gate_x_strides", ctypes.c_int64 * 2), ("gate_w", c_void_p)]
 
 
 # name -> (restype, argtypes); must list every symbol include/we_attn.h declares

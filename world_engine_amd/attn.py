@@ -133,8 +133,8 @@ class RingAttn(nn.Module):
     patch (``src/patch_model.py:102-114``); otherwise the keys are ``q_proj/k_proj/v_proj``.
 
     ``fuse_elementwise`` moves the module's element-wise neighbours of the attention (QK RMS
-    norm, value-residual lerp, head gate) into the two kernels: five to seven launches fewer per
-    layer, results within 1 ulp of the separate torch operations instead of bit-identical, which
+    norm, value-residual lerp, head gate incl. its H x H projection and sigmoid) into the two
+    kernels: seven to nine launches fewer per layer, results within 1 ulp of the separate torch operations instead of bit-identical, which
     is why it is off unless asked for.
     """
 
@@ -208,11 +208,13 @@ class RingAttn(nn.Module):
             elif not first:                      # lerp(v, v, w) is v
                 extras.update(v1=v1.view_as(v), v_lamb=self.v_lamb)
 
-        gates = torch.sigmoid(self.gate_proj(x[..., : self.n_heads])) if self.gated_attn else None
+        gates = None
+        if self.gated_attn and not fuse:
+            gates = torch.sigmoid(self.gate_proj(x[..., : self.n_heads]))
         if fuse:
             extras["qk_norm_eps"] = torch.finfo(torch.float32).eps     # F.rms_norm's epsilon for these inputs
-            if gates is not None:
-                extras["gate"] = gates.permute(0, 2, 1)
+            if self.gated_attn:      # projection + sigmoid + multiply all happen in the kernels' epilogues
+                extras.update(gate_x=x[..., : self.n_heads], gate_w=self.gate_proj.weight)
         else:
             q = F.rms_norm(q, (self.d_head,))
             k = F.rms_norm(k, (self.d_head,))

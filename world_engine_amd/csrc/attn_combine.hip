@@ -60,8 +60,8 @@ __global__ void __launch_bounds__(256) attn_combine_kernel(AttnParams p) {
   uint16_t* dst = reinterpret_cast<uint16_t*>(p.out) + b * p.os_b + h * p.os_h + (int64_t)t * p.os_t + dg * 8;
   frag_t y = M::pack8(acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv, acc[4] * inv, acc[5] * inv,
                       acc[6] * inv, acc[7] * inv);
-  if (p.gate != nullptr) {  // y * gate on element-type values, as the module's own multiply
-    const float g = (float)reinterpret_cast<const typename M::elem_t*>(p.gate)[b * p.gs_b + h * p.gs_h + (int64_t)t * p.gs_t];
+  if (p.gate != nullptr || p.gate_w != nullptr) {  // y * gate on element-type values, as the module's own multiply
+    const float g = head_gate<typename M::elem_t>(p, b, h, t);
     y = M::pack8((float)y[0] * g, (float)y[1] * g, (float)y[2] * g, (float)y[3] * g, (float)y[4] * g,
                  (float)y[5] * g, (float)y[6] * g, (float)y[7] * g);
   }

@@ -58,4 +58,20 @@ __device__ __forceinline__ void half_wave_pair(float x, float& lower, float& upp
 
 typedef __attribute__((address_space(3))) s16x4_t* lds_s16x4_ptr;
 
+// Head gate of output row (b, h, t): the given value, or sigmoid(gate_proj(x[b, t, :H]))[h] with
+// the module's rounding steps (src/model/attn.py:117-118: the projection's output and the sigmoid's
+// are both element-type tensors).  The dot product runs in fp32 in channel order.
+template <typename E, typename P>
+__device__ __forceinline__ float head_gate(const P& p, int b, int h, int64_t t) {
+  if (p.gate_w != nullptr) {
+    const E* x = reinterpret_cast<const E*>(p.gate_x) + b * p.gx_b + t * p.gx_t;
+    const E* w = reinterpret_cast<const E*>(p.gate_w) + (int64_t)h * p.H;
+    float acc = 0.f;
+    for (int j = 0; j < p.H; ++j) acc = __builtin_fmaf((float)x[j], (float)w[j], acc);
+    const float pre = (float)(E)acc;
+    return (float)(E)(1.f / (1.f + __expf(-pre)));
+  }
+  return (float)reinterpret_cast<const E*>(p.gate)[b * p.gs_b + h * p.gs_h + t * p.gs_t];
+}
+
 }  // namespace we

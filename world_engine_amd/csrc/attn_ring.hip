@@ -662,8 +662,8 @@ attn_ring_kernel(AttnParams p) {
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   const int64_t row = ((int64_t)b * p.H + h) * p.T + qrow;
   float gate_v = 1.f;
-  if (p.gate != nullptr && nsp == 1 && qrow < p.T)
-    gate_v = (float)reinterpret_cast<const typename M::elem_t*>(p.gate)[b * p.gs_b + h * p.gs_h + (int64_t)qrow * p.gs_t];
+  const bool gated = p.gate != nullptr || p.gate_w != nullptr;
+  if (gated && nsp == 1 && qrow < p.T) gate_v = head_gate<typename M::elem_t>(p, b, h, qrow);
   // A split leaves its partial output as fp16 values in [-1, 1] plus one fp32 scale per row (the
   // row's largest normalised magnitude): 11 significant bits whatever the element type, for the
   // bytes of a bf16 row, and no overflow whatever V holds.
@@ -702,7 +702,7 @@ attn_ring_kernel(AttnParams p) {
           uint16_t* dst = reinterpret_cast<uint16_t*>(p.out) + b * p.os_b + h * p.os_h +
                           (int64_t)qrow * p.os_t + d0;
           frag_t y = M::pack8(f[0], f[1], f[2], f[3], f[4], f[5], f[6], f[7]);
-          if (p.gate != nullptr) {  // y * gate on element-type values, as the module's own multiply
+          if (gated) {  // y * gate on element-type values, as the module's own multiply
             y = M::pack8((float)y[0] * gate_v, (float)y[1] * gate_v, (float)y[2] * gate_v, (float)y[3] * gate_v,
                          (float)y[4] * gate_v, (float)y[5] * gate_v, (float)y[6] * gate_v, (float)y[7] * gate_v);
           }

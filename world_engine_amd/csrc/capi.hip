@@ -195,6 +195,7 @@ int prepare_attn(const void* q, const int64_t* q_strides, const void* kv, const 
   p.unit_splits = pl.units_whole + (B * Hkv - pl.units_whole) * pl.n_splits;
   p.scale_log2 = scale * 1.4426950408889634f;
   p.gate = nullptr; p.gs_b = p.gs_h = p.gs_t = 0;
+  p.gate_x = nullptr; p.gate_w = nullptr; p.gx_b = p.gx_t = 0;
   p.clock_out = nullptr;
 
   if ((p.unit_splits + 7) / 8 > 65535 || p.group > 65535 || (int64_t)B * H - (int64_t)pl.units_whole * p.group > 65535)
@@ -379,8 +380,12 @@ int we_rope_kv_attn_fwd(const void* q, const void* k, const void* v, const int64
     sp.norm_eps = x.qk_norm_eps;
     sp.v1 = x.v1; sp.v_lamb = x.v_lamb;
     sp.v1s_b = x.v1_strides[0]; sp.v1s_h = x.v1_strides[1]; sp.v1s_t = x.v1_strides[2];
+    if ((x.gate_x == nullptr) != (x.gate_w == nullptr)) return WE_ERR_NULL_POINTER;
+    if (x.gate_w != nullptr && (x.gate != nullptr || dtype == WE_DTYPE_F32)) return WE_ERR_UNSUPPORTED;
     p.gate = x.gate;
     p.gs_b = x.gate_strides[0]; p.gs_h = x.gate_strides[1]; p.gs_t = x.gate_strides[2];
+    p.gate_x = x.gate_x; p.gate_w = x.gate_w;
+    p.gx_b = x.gate_x_strides[0]; p.gx_t = x.gate_x_strides[1];
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
   // Everything is validated before the first launch; the kernels follow each other on the stream.

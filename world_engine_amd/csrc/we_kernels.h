@@ -56,9 +56,13 @@ struct AttnParams {
   int members;      // workgroups that share one K/V stream: group * q_tiles
   int unit_splits;  // units_whole + (B * Hkv - units_whole) * n_splits
   float scale_log2;  // softmax scale * log2(e), applied to the raw logits in fp32
-  // optional per (batch, head, token) output gate, element type (src/model/attn.py:117-119)
+  // optional per (batch, head, token) output gate, element type (src/model/attn.py:117-119): either
+  // given (sigmoid applied), or computed here from the module's input and gate_proj.weight
   const void* gate;
   int64_t gs_b, gs_h, gs_t;
+  const void* gate_x;   // x[b, t, 0:H], channel stride 1, element strides gx_b / gx_t (null: no projection here)
+  const void* gate_w;   // gate_proj.weight [H, H] row-major (out, in), element type
+  int64_t gx_b, gx_t;
   // measurement aid (null = off): every workgroup of the main kernel leaves its duration as
   // (shader-clock cycles, ticks of the constant 100 MHz counter) at [2 * linear workgroup id]
   uint64_t* clock_out;

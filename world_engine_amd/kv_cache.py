@@ -118,7 +118,8 @@ class LayerKVCache(nn.Module):
     def rope_upsert_attend(self, q: Tensor, k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor], rope,
                            is_frozen: bool, scale: Optional[float] = None, qk_norm_eps: float = 0.0,
                            v1: Optional[Tensor] = None, v_lamb: Optional[Tensor] = None,
-                           gate: Optional[Tensor] = None) -> Tensor:
+                           gate: Optional[Tensor] = None, gate_x: Optional[Tensor] = None,
+                           gate_w: Optional[Tensor] = None) -> Tensor:
         """``rope_upsert`` followed by the attention over the ring, as one library call
         (``src/model/attn.py:110-116`` of the reference from RoPE to ``flex_attention``).  Under
         ``torch.compile`` the registered opaque op is used instead of the eager wrapper."""
@@ -127,11 +128,12 @@ class LayerKVCache(nn.Module):
             return torch.ops.world_engine_amd.rope_kv_attn(
                 q, k, v, pos_ids["t_pos"], pos_ids["y_pos"], pos_ids["x_pos"], rope.cos, rope.sin, rope.height,
                 rope.width, self.kv, self.written, self.L, self.pinned_dilation, bool(is_frozen), s,
-                float(qk_norm_eps), v1, v_lamb, gate)
+                float(qk_norm_eps), v1, v_lamb, gate, gate_x, gate_w)
         self._check(k, pos_ids, rope)
         return ops.rope_kv_attn(q, k, v, pos_ids, rope.cos, rope.sin, rope.height, rope.width, self.kv,
                                 self.written, self.L, self.pinned_dilation, is_frozen, scale,
-                                qk_norm_eps=qk_norm_eps, v1=v1, v_lamb=v_lamb, gate=gate)[0]
+                                qk_norm_eps=qk_norm_eps, v1=v1, v_lamb=v_lamb, gate=gate, gate_x=gate_x,
+                                gate_w=gate_w)[0]
 
 
 class StaticKVCache(nn.Module):

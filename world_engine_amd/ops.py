@@ -44,6 +44,16 @@ def _stream_ptr(dev: torch.device) -> int:
     return torch.cuda.current_stream(dev).cuda_stream
 
 
+def _call(dev: torch.device, fn, *args):
+    """Call a library entry point with the tensors' device current: the library configures and
+    launches its kernels on the device that is current when it is called (per-device LDS limits,
+    the static scratch buffer's address).  No overhead when it already is."""
+    if dev.index == torch.cuda.current_device():
+        return fn(*args)
+    with torch.cuda.device(dev):
+        return fn(*args)
+
+
 def _bhtd_strides(t: Tensor, what: str):
     if t.dim() != 4 or t.stride(3) != 1:
         raise RuntimeError(f"{what} must be [B, H, T, Dh] with a contiguous last dimension")
@@ -115,7 +125,8 @@ def rope_kv_store(q: Optional[Tensor], k: Tensor, v: Tensor, pos_ids: Mapping[st
     if rotate:
         _check_tables(cos_table, sin_table, Dh)
     t_pos, y_pos, x_pos, ps = _pos_triplet(pos_ids, B, T, rotate)
-    code = _capi.lib().we_rope_kv_store(
+    code = _call(
+        dev, _capi.lib().we_rope_kv_store,
         q.data_ptr() if q is not None else None, k.data_ptr(), v.data_ptr(),
         _bhtd_strides(q, "q") if q is not None else None, _bhtd_strides(k, "k"), _bhtd_strides(v, "v"),
         q_out.data_ptr() if q_out is not None else None,
@@ -141,7 +152,8 @@ def rope_apply(x: Tensor, pos_ids: Mapping[str, Tensor], cos_table: Tensor, sin_
         raise RuntimeError("cos/sin tables must be [rows, Dh/2]")
     t_pos, y_pos, x_pos, ps = _pos_triplet(pos_ids, B, T, True)
     out = torch.empty((B, H, T, Dh), dtype=x.dtype, device=dev)
-    code = _capi.lib().we_rope_apply(
+    code = _call(
+        dev, _capi.lib().we_rope_apply,
         x.data_ptr(), _bhtd_strides(x, "x"), out.data_ptr(),
         cos_table.contiguous().data_ptr(), sin_table.contiguous().data_ptr(), cos_table.shape[0],
         t_pos.data_ptr(), y_pos.data_ptr(), x_pos.data_ptr(), ps, grid_h, grid_w,
@@ -207,10 +219,10 @@ def attn_ring(q: Tensor, kv: Tensor, written: Tensor, t_pos: Tensor, L: int, dil
     if clocks is not None:
         if clocks.dtype != torch.int64 or not clocks.is_contiguous() or clocks.device != dev:
             raise RuntimeError("clocks must be a contiguous int64 tensor on q's device")
-        code = lib.we_attn_ring_fwd_clocked(*common, clocks.data_ptr(), clocks.numel(), _stream_ptr(dev))
+        code = _call(dev, lib.we_attn_ring_fwd_clocked, *common, clocks.data_ptr(), clocks.numel(), _stream_ptr(dev))
         _capi.check(code, "we_attn_ring_fwd_clocked")
     else:
-        code = lib.we_attn_ring_fwd(*common, _stream_ptr(dev))
+        code = _call(dev, lib.we_attn_ring_fwd, *common, _stream_ptr(dev))
         _capi.check(code, "we_attn_ring_fwd")
     return out
 
@@ -237,11 +249,11 @@ def attn_ring_static(q: Tensor, kv: Tensor, written: Tensor, t_pos: Tensor, L: i
     if tuple(out.shape) != (B, H, T, Dh) or out.dtype != q.dtype:
         raise RuntimeError("out must be [B, H, T, Dh] of q's element type on q's device")
     scale = 1.0 / math.sqrt(Dh) if scale is None else float(scale)
-    with torch.cuda.device(dev):     # the buffer's address is per device: the call must see q's device as current
-        code = _capi.lib().we_attn_ring_fwd_static(
-            q.data_ptr(), _bhtd_strides(q, "q"), kv.data_ptr(), written.data_ptr(), t_pos.data_ptr(),
-            out.data_ptr(), _bhtd_strides(out, "out"), B, H, kv.shape[2], T, Dh, L, dilation, scale, n_splits, q_tile,
-            _dtype_code(q), _stream_ptr(dev))
+    code = _call(   # (the buffer's address is per device: the call must see q's device as current)
+        dev, _capi.lib().we_attn_ring_fwd_static,
+        q.data_ptr(), _bhtd_strides(q, "q"), kv.data_ptr(), written.data_ptr(), t_pos.data_ptr(),
+        out.data_ptr(), _bhtd_strides(out, "out"), B, H, kv.shape[2], T, Dh, L, dilation, scale, n_splits, q_tile,
+        _dtype_code(q), _stream_ptr(dev))
     _capi.check(code, "we_attn_ring_fwd_static")
     return out
 
@@ -251,7 +263,8 @@ def rope_kv_attn(q: Tensor, k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor],
                  dilation: int, is_frozen: bool, scale: Optional[float] = None, n_splits: int = 0,
                  q_tile: int = 0, out: Optional[Tensor] = None, workspace: Optional[Tensor] = None,
                  token_major_out: bool = True, qk_norm_eps: float = 0.0, v1: Optional[Tensor] = None,
-                 v_lamb: Optional[Tensor] = None, gate: Optional[Tensor] = None):
+                 v_lamb: Optional[Tensor] = None, gate: Optional[Tensor] = None,
+                 gate_x: Optional[Tensor] = None, gate_w: Optional[Tensor] = None):
     """``rope_kv_store`` followed by ``attn_ring`` in one library call (``we_rope_kv_attn_fwd``):
     the per-layer sequence of the reference from ``q, k = rope(q), rope(k)`` to the
     ``flex_attention`` call (``src/model/attn.py:110-116``), validated as a whole before the first
@@ -289,7 +302,7 @@ def rope_kv_attn(q: Tensor, k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor],
     elif tuple(out.shape) != (B, H, T, Dh) or out.dtype != q.dtype or out.device != dev:
         raise RuntimeError("out must be [B, H, T, Dh] of q's element type on q's device")
     extras = None
-    if qk_norm_eps or v1 is not None or gate is not None:
+    if qk_norm_eps or v1 is not None or gate is not None or gate_w is not None:
         ex = _capi.AttnExtras()
         ex.qk_norm_eps = float(qk_norm_eps)
         if v1 is not None:
@@ -304,8 +317,20 @@ def rope_kv_attn(q: Tensor, k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor],
             _need_device(gate)
             ex.gate = gate.data_ptr()
             ex.gate_strides = _capi.i64x3(*gate.stride())
+        if gate_w is not None:
+            if gate is not None:
+                raise RuntimeError("give either gate or gate_x / gate_w")
+            if (gate_x is None or gate_x.dim() != 3 or tuple(gate_x.shape) != (B, T, H) or gate_x.stride(2) != 1
+                    or gate_x.dtype != q.dtype or tuple(gate_w.shape) != (H, H) or gate_w.dtype != q.dtype
+                    or not gate_w.is_contiguous()):
+                raise RuntimeError("gate_x must be [B, T, H] (contiguous channels) and gate_w a contiguous [H, H], "
+                                   "both of q's element type")
+            _need_device(gate_x, gate_w)
+            ex.gate_x, ex.gate_w = gate_x.data_ptr(), gate_w.data_ptr()
+            ex.gate_x_strides = (ctypes.c_int64 * 2)(gate_x.stride(0), gate_x.stride(1))
         extras = ctypes.byref(ex)
-    code = lib.we_rope_kv_attn_fwd(
+    code = _call(
+        dev, lib.we_rope_kv_attn_fwd,
         q.data_ptr(), k.data_ptr(), v.data_ptr(), _bhtd_strides(q, "q"), _bhtd_strides(k, "k"), _bhtd_strides(v, "v"),
         q_rot.data_ptr(), cos_table.data_ptr(), sin_table.data_ptr(), cos_table.shape[0],
         t_pos.data_ptr(), y_pos.data_ptr(), x_pos.data_ptr(), ps, grid_h, grid_w, kv.data_ptr(), written.data_ptr(),
@@ -354,14 +379,17 @@ def rope_kv_attn_op(q: Tensor, k: Tensor, v: Tensor, t_pos: Tensor, y_pos: Tenso
                     cos_table: Tensor, sin_table: Tensor, grid_h: int, grid_w: int,
                     kv: Tensor, written: Tensor, L: int, dilation: int, is_frozen: bool, scale: float,
                     qk_norm_eps: float = 0.0, v1: Optional[Tensor] = None, v_lamb: Optional[Tensor] = None,
-                    gate: Optional[Tensor] = None) -> Tensor:
+                    gate: Optional[Tensor] = None, gate_x: Optional[Tensor] = None,
+                    gate_w: Optional[Tensor] = None) -> Tensor:
     pos = {"t_pos": t_pos, "y_pos": y_pos, "x_pos": x_pos}
     return rope_kv_attn(q, k, v, pos, cos_table, sin_table, grid_h, grid_w, kv, written, L, dilation,
-                        is_frozen, scale, qk_norm_eps=qk_norm_eps, v1=v1, v_lamb=v_lamb, gate=gate)[0]
+                        is_frozen, scale, qk_norm_eps=qk_norm_eps, v1=v1, v_lamb=v_lamb, gate=gate,
+                        gate_x=gate_x, gate_w=gate_w)[0]
 
 
 @rope_kv_attn_op.register_fake
 def _rope_kv_attn_fake(q, k, v, t_pos, y_pos, x_pos, cos_table, sin_table, grid_h, grid_w, kv, written, L,
-                       dilation, is_frozen, scale, qk_norm_eps=0.0, v1=None, v_lamb=None, gate=None):
+                       dilation, is_frozen, scale, qk_norm_eps=0.0, v1=None, v_lamb=None, gate=None, gate_x=None,
+                       gate_w=None):
     B, H, T, Dh = q.shape
     return q.new_empty((B, T, H, Dh)).transpose(1, 2)
