@@ -339,6 +339,35 @@ def test_output_layout_and_out_argument(gpu_device):
     assert c.data_ptr() == out.data_ptr() and torch.equal(out, b)
 
 
+def test_clocked_entry_point_same_output_and_plausible_clocks(gpu_device):
+    """``we_attn_ring_fwd_clocked`` is ``we_attn_ring_fwd`` plus two counters per workgroup: the
+    output has the same bits, every workgroup reports a duration, and cycles per 100 MHz tick is a
+    shader frequency the part can run at."""
+    p = Pair(gpu_device, torch.bfloat16, B=1, H=4, Hkv=2, T=128, Dh=128, n_slots=4, cfg_id=27)
+    p.set_frozen(False)
+    for t in range(5):
+        q, k, v, pos = p.inputs(t)
+        (q_o, k_all, v_all, mask), (q_h, ring) = p.store(q, k, v, pos)
+    plain = p.attend(q_h, ring, n_splits=2)
+    assert_attn_close(plain, ro.attention_fp32(q_o, k_all, v_all, mask), "plain")
+    clocks = torch.zeros(2 * 1024, dtype=torch.int64, device=gpu_device)
+    timed = p.attend(q_h, ring, n_splits=2, clocks=clocks)
+    assert_bits_equal(timed, plain, "clocked output")
+    c = clocks.view(-1, 2).cpu()
+    c = c[c[:, 0] != 0]
+    _say(f"clocked: {c.shape[0]} workgroups, cycles {c[:4, 0].tolist()} ticks {c[:4, 1].tolist()}")
+    # 1 query tile x 2 query heads per kv head x (2 kv heads x 2 context parts); grid slots past
+    # the last part leave early and report nothing
+    assert c.shape[0] == 1 * 2 * (2 * 2), "one report per working workgroup"
+    assert torch.all(c[:, 1] > 0)
+    ghz = (c[:, 0].double() / c[:, 1].double()).median().item() * 0.1
+    assert 0.3 < ghz < 3.0, f"implausible shader clock {ghz} GHz"
+    with pytest.raises(RuntimeError, match="we_attn_ring_fwd_clocked"):
+        p.attend(q_h, ring, n_splits=2, clocks=clocks[:2])
+    with pytest.raises(RuntimeError, match="int64"):
+        p.attend(q_h, ring, n_splits=2, clocks=clocks.to(torch.int32))
+
+
 # ------------------------------------------------------------------------------------------
 # module-level drop-in and graph capture
 # ------------------------------------------------------------------------------------------
