@@ -261,6 +261,68 @@ int we_rope_kv_attn_fwd(const void* q, const void* k, const void* v,
                         int32_t dilation, int32_t is_frozen, float scale, int32_t n_splits, int32_t q_tile,
                         int32_t dtype, const we_attn_extras* extras, void* stream);
 
+/*
+ * The module's merged q/k/v projection as the producer of the path (next-row 3 of the scope:
+ * `q, k, v = self.qkv_proj(x).split(...)`, src/patch_model.py:116-122, weights merged as in
+ * :102-114).  Describes the GEMM operands for we_qkv_rope_kv_store / we_qkv_rope_kv_attn_fwd:
+ *   x            module input [B, T, d_model], channel stride 1, element strides x_strides =
+ *                {batch, token} (multiples of 8), 16-byte aligned.
+ *   w            qkv_proj.weight [(H + 2 Hkv) * Dh, d_model] row-major (out, in): q rows, then k
+ *                rows, then v rows; element stride w_row_stride between rows (multiple of 8).
+ *   d_model      contraction length, a multiple of 128.
+ *   v_out        optional: the projected v rows as the GEMM leaves them (before the value blend),
+ *                [B, Hkv, T, Dh] with element strides v_out_strides = {batch, head, token} - what
+ *                the first layer hands on as `v1` (src/model/attn.py:107).  NULL = not wanted.
+ * The projection accumulates in fp32 and rounds once to the element type, like the GEMM's output
+ * tensor; sums are taken in a fixed order (results are reproducible, and exact whenever the fp32
+ * sums are exact) that differs from a BLAS library's, i.e. rows may differ from
+ * torch.nn.functional.linear's in the last bit of the element type.  bf16 / f16 only;
+ * (H + 2 Hkv) * Dh must be a multiple of 128 and Dh 64 or 128.
+ */
+typedef struct we_qkv_proj {
+  const void* x;
+  int64_t x_strides[2];
+  const void* w;
+  int64_t w_row_stride;
+  int32_t d_model;
+  void* v_out;
+  int64_t v_out_strides[3];
+} we_qkv_proj;
+
+/*
+ * we_rope_kv_store with the projection in front, in one kernel: computes q, k, v = x W^T tile by
+ * tile on the matrix cores and applies the store's work (optional RMS norm and value blend from
+ * `extras`, RoPE, q_out, tail / ring-slot rows, `written`) to each tile while it is still on the
+ * CU; the [B, T, (H + 2 Hkv) Dh] projection output never exists in memory.  Arguments other than
+ * `proj` are those of we_rope_kv_store (q_out and the tables may not be NULL); of `extras` only
+ * qk_norm_eps, v1 and v_lamb are used.  Replaces src/patch_model.py:116-122 +
+ * src/model/attn.py:105-110 + src/model/kv_cache.py:126-151,192.
+ */
+int we_qkv_rope_kv_store(const we_qkv_proj* proj, void* q_out,
+                         const float* cos_table, const float* sin_table, int64_t table_rows,
+                         const int64_t* t_pos, const int64_t* y_pos, const int64_t* x_pos,
+                         int64_t pos_stride_b, int64_t grid_h, int64_t grid_w,
+                         void* kv, uint8_t* written,
+                         int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L,
+                         int32_t dilation, int32_t is_frozen, int32_t dtype,
+                         const we_attn_extras* extras, void* stream);
+
+/*
+ * we_rope_kv_attn_fwd with the projection in front: we_qkv_rope_kv_store, then we_attn_ring_fwd on
+ * the rotated q (two or three launches for everything between the module's input and out_proj).
+ * Both are validated before anything is launched.
+ */
+int we_qkv_rope_kv_attn_fwd(const we_qkv_proj* proj, void* q_out,
+                            const float* cos_table, const float* sin_table, int64_t table_rows,
+                            const int64_t* t_pos, const int64_t* y_pos, const int64_t* x_pos,
+                            int64_t pos_stride_b, int64_t grid_h, int64_t grid_w,
+                            void* kv, uint8_t* written,
+                            void* out, const int64_t out_strides[3],
+                            void* workspace, size_t workspace_bytes,
+                            int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L,
+                            int32_t dilation, int32_t is_frozen, float scale, int32_t n_splits, int32_t q_tile,
+                            int32_t dtype, const we_attn_extras* extras, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

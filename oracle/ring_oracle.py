@@ -17,6 +17,8 @@ Reference sources followed (paths relative to the world_engine checkout):
 * ``src/model/attn.py:99-122`` / ``src/patch_model.py:116-141``  order of operations, incl. the
   module's element-wise steps around the path: value-residual lerp (``attn.py:105-107``), weightless
   QK RMS norm (``attn.py:109``, ``src/model/nn.py:55-56``), sigmoid head gate (``attn.py:117-119``)
+* ``src/patch_model.py:102-122``    merged q/k/v projection in front of the path (weight rows q | k | v,
+  split, ``[B,T,H,Dh] -> [B,H,T,Dh]`` views)
 * ``src/world_engine.py:139-152``   frozen denoise passes followed by one unfrozen cache pass
 * ``torch/_higher_order_ops/flex_attention.py:159-267`` (torch 2.10, third-party) dtype flow
   of eager ``flex_attention``: fp32 scores, ``* scale``, ``where(mask, s, -inf)``, softmax,
@@ -37,6 +39,10 @@ Pinning status (see tests/test_oracle_pins.py; the reference ships no tests or g
 * ``rms_norm`` / ``value_lerp`` / ``gate_output``  pinned: torch's own ``F.rms_norm`` / ``torch.lerp``
   (library routines, the calls the reference makes) bit for bit on the CPU, plus closed cases
   (unit RMS, power-of-two scale invariance, lerp end points, gate 0 / 1)
+* ``qkv_project``                    pinned: exact integer arithmetic on dyadic inputs (every
+  summation order gives the same fp32 sum there), fp64 sums rounded once on random inputs
+  (within one unit in the last place), torch's own ``F.linear`` + the reference's
+  split / reshape / transpose for the layout
 * ``rope_table_1d``                  synthetic table of the benchmark configurations (not a
   reference function); checked against direct fp64 evaluation
 * ``ortho_rope_table``               parity unpinned: depends on ``rotary_embedding_torch``
@@ -322,6 +328,25 @@ def gate_output(y: Tensor, gates: Tensor) -> Tensor:
 
 
 # --------------------------------------------------------------------------------------
+# the merged projection in front of the path              src/patch_model.py:102-122
+# --------------------------------------------------------------------------------------
+def qkv_project(x: Tensor, w_qkv: Tensor, n_heads: int, n_kv_heads: int) -> Tuple[Tensor, Tensor, Tensor]:
+    """``q, k, v = self.qkv_proj(x).split((H Dh, Hkv Dh, Hkv Dh), dim=-1)`` followed by the
+    ``[B,T,h,Dh] -> [B,h,T,Dh]`` views (src/patch_model.py:116-122; the weight's rows are the q,
+    k and v projections' rows one after the other, :102-114).  A bias-free linear layer of the
+    element type: every output is the fp32 sum of the products, rounded once to ``x``'s dtype.
+    The order of the fp32 additions is the BLAS library's business in the reference; here it is
+    torch's CPU matmul on fp32 copies."""
+    B, T, _ = x.shape
+    d_head = w_qkv.shape[0] // (n_heads + 2 * n_kv_heads)
+    wp = torch.float64 if x.dtype == torch.float64 else torch.float32
+    y = (x.to(wp) @ w_qkv.to(wp).t()).to(x.dtype)
+    q, k, v = y.split((n_heads * d_head, n_kv_heads * d_head, n_kv_heads * d_head), dim=-1)
+    return (q.reshape(B, T, n_heads, d_head).transpose(1, 2), k.reshape(B, T, n_kv_heads, d_head).transpose(1, 2),
+            v.reshape(B, T, n_kv_heads, d_head).transpose(1, 2))
+
+
+# --------------------------------------------------------------------------------------
 # one attention-layer step in the reference's order of operations
 #                                  src/model/attn.py:105-119, src/patch_model.py:124-137
 # --------------------------------------------------------------------------------------
@@ -366,6 +391,17 @@ def synth_qkv(cfg_id: int, step: int, substep: int, B: int, H: int, Hkv: int, T:
         ch = int(torch.randint(0, Dh, (1,), generator=g))
         k[..., ch] *= 8.0
     return q.to(dtype), k.to(dtype), v.to(dtype)
+
+
+def synth_dyadic_linear(seed: int, B: int, T: int, d_model: int, feats: int,
+                        dtype: torch.dtype) -> Tuple[Tensor, Tensor]:
+    """x ``[B,T,d_model]`` and w ``[feats,d_model]`` whose values are multiples of 1/8 in [-1, 1]:
+    every product is a multiple of 1/64 and every partial sum of up to 2^17 of them is an exact
+    fp32 number, so a linear layer's fp32 sums do not depend on the order of the additions."""
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    x = (torch.randint(-8, 9, (B, T, d_model), generator=g).float() / 8).to(dtype)
+    w = (torch.randint(-8, 9, (feats, d_model), generator=g).float() / 8).to(dtype)
+    return x, w
 
 
 def synth_pos_ids(frame_t: int, B: int, T: int, width: int) -> Dict[str, Tensor]:

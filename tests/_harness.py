@@ -108,3 +108,15 @@ def assert_attn_close(out_hip: torch.Tensor, ref32: torch.Tensor, what=""):
     assert math.isfinite(mx), f"non-finite output {what}"
     assert mx <= MAX_ABS and mean <= MEAN_ABS, f"{what}: max-abs {mx:.3e} (<= {MAX_ABS}), mean-abs {mean:.3e} (<= {MEAN_ABS})"
     return mx, mean
+
+
+def assert_ulp_close(a, b, what, ulps=1):
+    """Element-type tensors equal up to `ulps` units in the last place of the largest value of
+    their row (a last-bit difference in a normalised input moves a rotated pair, a difference of
+    products, by that much whatever the size of the result).  Returns the fraction that differs."""
+    a32, b32 = a.float().cpu(), b.float().cpu()
+    eps = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}[a.dtype]
+    tol = 2 * ulps * eps * b32.abs().amax(dim=-1, keepdim=True).clamp_min(2.0 ** -100)
+    bad = (a32 - b32).abs() > tol
+    assert not bad.any(), f"{what}: {int(bad.sum())} elements off by more than {ulps} ulp of their row's largest"
+    return float((a32 != b32).float().mean())

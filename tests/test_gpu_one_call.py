@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from oracle import ring_oracle as ro
-from _harness import Pair, assert_attn_close, assert_bits_equal, merged_views, to_dev
+from _harness import Pair, assert_attn_close, assert_bits_equal, assert_ulp_close, merged_views, to_dev
 from world_engine_amd import ops
 
 pytestmark = pytest.mark.gpu
@@ -118,18 +118,6 @@ def test_module_forward_compiles_as_one_graph(gpu_device, backend, fuse):
         assert torch.equal(caches[0].layers[0].written, caches[1].layers[0].written)
 
 
-def _ulp_close(a, b, what, ulps=1):
-    """Element-type tensors equal up to `ulps` units in the last place of the largest value of
-    their row (a last-bit difference in a normalised input moves a rotated pair, a difference of
-    products, by that much whatever the size of the result).  Returns the fraction that differs."""
-    a32, b32 = a.float().cpu(), b.float().cpu()
-    eps = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}[a.dtype]
-    tol = 2 * ulps * eps * b32.abs().amax(dim=-1, keepdim=True).clamp_min(2.0 ** -100)
-    bad = (a32 - b32).abs() > tol
-    assert not bad.any(), f"{what}: {int(bad.sum())} elements off by more than {ulps} ulp of their row's largest"
-    return float((a32 != b32).float().mean())
-
-
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_fused_neighbours_match_torch_ops(gpu_device, dtype):
     """qk RMS norm, value-residual lerp and head gate inside the kernels against the same torch
@@ -160,8 +148,8 @@ def test_fused_neighbours_match_torch_ops(gpu_device, dtype):
         out_u, qrot_u = ops.rope_kv_attn(qn, kn, vl, posd, p_u.rope.cos, p_u.rope.sin, p_u.rope.height, p_u.rope.width,
                                          lu.kv, lu.written, lu.L, 1, frozen)
         out_u = out_u * gate.unsqueeze(-1)
-        frac = _ulp_close(qrot_f, qrot_u, f"RoPE(norm(q)) t={t}")
-        frac_kv = _ulp_close(lf.kv, lu.kv, f"cache t={t}")
+        frac = assert_ulp_close(qrot_f, qrot_u, f"RoPE(norm(q)) t={t}")
+        frac_kv = assert_ulp_close(lf.kv, lu.kv, f"cache t={t}")
         assert frac < 0.02 and frac_kv < 0.02, (frac, frac_kv)
         assert torch.equal(lf.written, lu.written)
         assert_attn_close(out_f, out_u.float().cpu(), f"gated output t={t}")
@@ -204,8 +192,8 @@ def test_fused_neighbours_match_the_oracle(gpu_device, dtype, gate_mode):
         out, qrot_h = ops.rope_kv_attn(qd, kd, vd, to_dev(pos, dev), p.rope.cos, p.rope.sin, p.rope.height, p.rope.width,
                                        layer.kv, layer.written, layer.L, 1, frozen, qk_norm_eps=eps, v1=v1.to(dev),
                                        v_lamb=lamb.to(dev), **gate_kw)
-        frac_q = _ulp_close(qrot_h, q_rot, f"RoPE(norm(q)) t={t}")
-        frac_kv = _ulp_close(layer.kv, p.oracle.layers[0].kv, f"cache t={t}")
+        frac_q = assert_ulp_close(qrot_h, q_rot, f"RoPE(norm(q)) t={t}")
+        frac_kv = assert_ulp_close(layer.kv, p.oracle.layers[0].kv, f"cache t={t}")
         assert frac_q < 0.02 and frac_kv < 0.02, (frac_q, frac_kv)
         assert torch.equal(layer.written.cpu(), p.oracle.layers[0].written)
         assert_attn_close(out, ref, f"gated output t={t}")
@@ -245,4 +233,4 @@ def test_module_with_fused_neighbours(gpu_device):
         scale = ya2.float().abs().max().item()
         assert d1 <= 2e-2 * max(1.0, ya.float().abs().max().item()) and d2 <= 3e-2 * max(1.0, scale), (t, d1, d2)
         for li in range(2):
-            _ulp_close(caches[1].layers[li].kv, caches[0].layers[li].kv, f"layer {li} cache t={t}", ulps=2 if li else 1)
+            assert_ulp_close(caches[1].layers[li].kv, caches[0].layers[li].kv, f"layer {li} cache t={t}", ulps=2 if li else 1)

@@ -1,0 +1,133 @@
+"""GPU parity of the merged q/k/v projection fused with RoPE + the K/V store
+(we_qkv_rope_kv_store / we_qkv_rope_kv_attn_fwd; src/patch_model.py:116-122 in front of
+src/model/attn.py:105-116).
+
+On dyadic operands (multiples of 1/8) every fp32 sum of the projection is exact whatever the
+order of the additions, so everything the kernel writes - RoPE(q), cache rows, ``written``, the
+projected v rows - must equal the oracle's bit for bit.  On random operands the projection may
+differ from the oracle's in the last bit of the element type (summation order), so rows are
+compared to 1 ulp of their largest value and the attention output to the usual 2e-2 / 2e-3.
+"""
+import pytest
+import torch
+
+from oracle import ring_oracle as ro
+from _harness import Pair, assert_attn_close, assert_bits_equal, assert_ulp_close, to_dev
+from world_engine_amd import ops
+
+pytestmark = pytest.mark.gpu
+
+
+def _operands(kind, seed, B, T, d_model, feats, dtype):
+    if kind == "dyadic":
+        return ro.synth_dyadic_linear(seed, B, T, d_model, feats, dtype)
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(B, T, d_model, generator=g).to(dtype)
+    w = (torch.randn(feats, d_model, generator=g) / d_model ** 0.5).to(dtype)
+    return x, w
+
+
+def _proj_step(p, t, frozen, x, w, attend=True, exact=True, **kw):
+    """One frame through the oracle (projection, then layer_step) and through the fused call."""
+    p.set_frozen(frozen)
+    pos = ro.synth_pos_ids(t, p.B, p.T, p.W)
+    q, k, v = ro.qkv_project(x, w, p.H, p.Hkv)
+    ref, q_o = ro.layer_step(p.oracle, 0, q, k, v, pos, p.cos, p.sin, p.Hgrid, p.W, reference_dtype_flow=False,
+                             qk_norm=bool(kw.get("qk_norm_eps")), v1=kw.get("v1"), v_lamb=kw.get("v_lamb"))
+    lay = p.hip.layers[0]
+    dkw = {k_: (v_.to(p.dev) if torch.is_tensor(v_) else v_) for k_, v_ in kw.items()}
+    out, q_rot, v_raw = ops.qkv_rope_kv_attn(x.to(p.dev), w.to(p.dev), p.H, p.Hkv, to_dev(pos, p.dev), p.rope.cos,
+                                             p.rope.sin, p.rope.height, p.rope.width, lay.kv, lay.written, lay.L,
+                                             lay.pinned_dilation, frozen, attend=attend, want_v=True, **dkw)
+    what = f"t={t} frozen={frozen}"
+    assert torch.equal(lay.written.cpu(), p.oracle.layers[0].written), f"written {what}"
+    if exact:
+        assert_bits_equal(q_rot, q_o, f"RoPE(q) {what}")
+        assert_bits_equal(v_raw, v, f"projected v {what}")
+        p.assert_state_equal(what=what)
+    else:
+        assert_ulp_close(q_rot, q_o, f"RoPE(q) {what}")
+        assert_ulp_close(v_raw, v, f"projected v {what}")
+        assert_ulp_close(lay.kv, p.oracle.layers[0].kv, f"cache {what}")
+    return out, ref
+
+
+@pytest.mark.parametrize("dtype,Dh,H,Hkv,T,B,d_model", [
+    (torch.bfloat16, 128, 4, 4, 128, 1, 256),
+    (torch.bfloat16, 128, 4, 2, 96, 2, 128),     # grouped heads, a short last token tile, one contraction step
+    (torch.float16, 128, 2, 2, 64, 1, 384),      # three contraction steps: the ring wraps exactly once
+    (torch.bfloat16, 64, 6, 2, 72, 2, 512),      # two heads per feature tile, 10 x 64 features
+    (torch.bfloat16, 64, 3, 1, 40, 1, 640),      # (H + 2 Hkv) Dh = 320 is not a whole number of feature tiles: refused
+])
+def test_projection_store_bit_exact_on_dyadic_operands(gpu_device, dtype, Dh, H, Hkv, T, B, d_model):
+    print(f"qkv store dtype={dtype} Dh={Dh} H={H} Hkv={Hkv} T={T} B={B} d_model={d_model}", flush=True)
+    feats = (H + 2 * Hkv) * Dh
+    p = Pair(gpu_device, dtype, B=B, H=H, Hkv=Hkv, T=T, Dh=Dh, n_slots=3, cfg_id=71)
+    if feats % 128 != 0:
+        x, w = ro.synth_dyadic_linear(0, B, T, d_model, feats, dtype)
+        with pytest.raises(RuntimeError, match="we_qkv_rope_kv_store"):
+            _proj_step(p, 0, False, x, w, attend=False)
+        return
+    for t in range(8):
+        x, w = ro.synth_dyadic_linear(100 * t + 1, B, T, d_model, feats, dtype)
+        _proj_step(p, t, t % 3 == 1, x, w, attend=False)
+
+
+def test_projection_attend_cfg1_shape(gpu_device):
+    """cfg1's module shapes (d_model 2048, 16 heads of 128, 256-token frames, 16-slot ring): exact
+    on dyadic operands, then random operands to 1 ulp and the attention bar."""
+    B, H, Hkv, T, Dh, d_model = 1, 16, 16, 256, 128, 2048
+    feats = (H + 2 * Hkv) * Dh
+    p = Pair(gpu_device, torch.bfloat16, B=B, H=H, Hkv=Hkv, T=T, Dh=Dh, n_slots=16, cfg_id=72)
+    for t in range(3):
+        print(f"cfg1 dyadic t={t}", flush=True)
+        x, w = ro.synth_dyadic_linear(200 + t, B, T, d_model, feats, torch.bfloat16)
+        out, ref = _proj_step(p, t, False, x, w)
+        # these v rows are sums of 2048 terms (magnitudes up to ~40, not ~4 as for unit-variance rows): the
+        # absolute bar is applied to outputs brought to unit scale by an exact power of two
+        assert_attn_close(out.float() / 16, ref / 16, f"dyadic t={t}")
+    p = Pair(gpu_device, torch.bfloat16, B=B, H=H, Hkv=Hkv, T=T, Dh=Dh, n_slots=16, cfg_id=73)
+    _, w = _operands("random", 300, B, T, d_model, feats, torch.bfloat16)
+    for t in list(range(4)) + [17, 18]:
+        print(f"cfg1 random t={t}", flush=True)
+        x, _ = _operands("random", 301 + t, B, T, d_model, feats, torch.bfloat16)
+        out, ref = _proj_step(p, t, t == 2, x, w, exact=False)
+        assert_attn_close(out, ref, f"random t={t}")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_projection_with_norm_and_value_blend(gpu_device, dtype):
+    """The store's optional steps behind the projection: weightless RMS norm of q and k rows and
+    the value blend, against the oracle's layer_step with the same steps (1 ulp of a row's largest
+    value, as for the store kernel); the projected v handed back is the one before the blend."""
+    B, H, Hkv, T, Dh, d_model = 2, 4, 2, 128, 128, 256
+    feats = (H + 2 * Hkv) * Dh
+    p = Pair(gpu_device, dtype, B=B, H=H, Hkv=Hkv, T=T, Dh=Dh, n_slots=3, cfg_id=74)
+    eps = torch.finfo(torch.float32).eps
+    g = torch.Generator().manual_seed(9)
+    lamb = torch.tensor(0.37, dtype=dtype)
+    for t in range(6):
+        print(f"norm+blend dtype={dtype} t={t}", flush=True)
+        x, w = ro.synth_dyadic_linear(400 + t, B, T, d_model, feats, dtype)
+        v1 = torch.randn(B, Hkv, T, Dh, generator=g).to(dtype)
+        out, ref = _proj_step(p, t, t % 3 == 1, x, w, exact=False, qk_norm_eps=eps, v1=v1, v_lamb=lamb)
+        assert_attn_close(out, ref, f"t={t}")
+
+
+def test_projection_rejects_bad_operands(gpu_device):
+    dev = gpu_device
+    p = Pair(dev, torch.bfloat16, B=1, H=2, Hkv=2, T=64, Dh=128, n_slots=2, cfg_id=75)
+    lay = p.hip.layers[0]
+    pos = to_dev(ro.synth_pos_ids(0, 1, 64, p.W), dev)
+    args = (p.rope.cos, p.rope.sin, p.rope.height, p.rope.width, lay.kv, lay.written, lay.L, 1, False)
+    x = torch.zeros(1, 64, 192, device=dev, dtype=torch.bfloat16)          # d_model not a multiple of 128
+    w = torch.zeros(6 * 128, 192, device=dev, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError):
+        ops.qkv_rope_kv_attn(x, w, 2, 2, pos, *args)
+    x = torch.zeros(1, 64, 256, device=dev, dtype=torch.bfloat16)
+    w = torch.zeros(5 * 128, 256, device=dev, dtype=torch.bfloat16)        # wrong number of weight rows
+    with pytest.raises(RuntimeError):
+        ops.qkv_rope_kv_attn(x, w, 2, 2, pos, *args)
+    before = lay.kv.clone()
+    torch.cuda.synchronize()
+    assert torch.equal(before, lay.kv)

@@ -432,3 +432,52 @@ def test_layer_step_with_module_steps_equals_their_composition():
         out_b = out_b * gates.permute(0, 2, 1).unsqueeze(-1)
         assert torch.equal(qa, qb) and torch.equal(out_a, out_b)
         assert torch.equal(a.layers[0].kv, b.layers[0].kv) and torch.equal(a.layers[0].written, b.layers[0].written)
+
+
+# ----------------------------------------------------------------------------------------
+# the merged q/k/v projection in front of the path
+# ----------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_qkv_project_exact_integer_case_and_layout(dtype):
+    """On dyadic operands the projection is integer arithmetic: the oracle must equal the int64
+    matrix product scaled by 1/64 and rounded once to the element type, and its q / k / v must be
+    the reference's views (src/patch_model.py:116-122) of that matrix - checked element by element
+    for the head / token / channel each output came from."""
+    B, T, d_model, H, Hkv, Dh = 2, 5, 96, 3, 1, 16
+    feats = (H + 2 * Hkv) * Dh
+    x, w = ro.synth_dyadic_linear(11, B, T, d_model, feats, dtype)
+    xi, wi = (x.double() * 8).long(), (w.double() * 8).long()
+    y = (torch.einsum("btk,nk->btn", xi, wi).double() / 64).to(dtype)          # exact, then one rounding
+    q, k, v = ro.qkv_project(x, w, H, Hkv)
+    assert q.shape == (B, H, T, Dh) and k.shape == (B, Hkv, T, Dh) and v.shape == (B, Hkv, T, Dh)
+    for b in range(B):
+        for t in range(T):
+            for h in range(H):
+                assert torch.equal(q[b, h, t], y[b, t, h * Dh:(h + 1) * Dh])
+            for h in range(Hkv):
+                assert torch.equal(k[b, h, t], y[b, t, (H + h) * Dh:(H + h + 1) * Dh])
+                assert torch.equal(v[b, h, t], y[b, t, (H + Hkv + h) * Dh:(H + Hkv + h + 1) * Dh])
+
+
+def test_qkv_project_matches_torch_linear_and_fp64():
+    """Against the call the reference makes (F.linear on element-type tensors, then split) and
+    against fp64 sums rounded once: identical on dyadic operands, within one unit in the last
+    place on random ones (the BLAS routine's summation order is not the oracle's)."""
+    import torch.nn.functional as F
+    B, T, d_model, H, Hkv, Dh = 1, 12, 256, 2, 2, 32
+    feats = (H + 2 * Hkv) * Dh
+    x, w = ro.synth_dyadic_linear(12, B, T, d_model, feats, torch.bfloat16)
+    q, k, v = ro.qkv_project(x, w, H, Hkv)
+    ql, kl, vl = F.linear(x, w).split((H * Dh, Hkv * Dh, Hkv * Dh), dim=-1)
+    assert torch.equal(q, ql.reshape(B, T, H, Dh).transpose(1, 2))
+    assert torch.equal(k, kl.reshape(B, T, Hkv, Dh).transpose(1, 2))
+    assert torch.equal(v, vl.reshape(B, T, Hkv, Dh).transpose(1, 2))
+    g = torch.Generator().manual_seed(13)
+    x = torch.randn(B, T, d_model, generator=g).to(torch.bfloat16)
+    w = (torch.randn(feats, d_model, generator=g) / 16).to(torch.bfloat16)
+    got = torch.cat([t_.transpose(1, 2).reshape(B, T, -1) for t_ in ro.qkv_project(x, w, H, Hkv)], dim=-1)
+    want64 = x.double() @ w.double().t()
+    ulp = 2.0 ** (torch.floor(torch.log2(want64.abs().clamp_min(1e-30))) - 7)       # bf16: 8 significant bits
+    assert ((got.double() - want64).abs() <= 0.5 * ulp + 1e-6 * want64.abs()).all()
+    lin = F.linear(x, w)
+    assert ((got.double() - lin.double()).abs() <= ulp).all()

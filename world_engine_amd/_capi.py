@@ -26,6 +26,12 @@ class AttnExtras(ctypes.Structure):
                 ("gate_x", c_void_p), ("gate_x_strides", ctypes.c_int64 * 2), ("gate_w", c_void_p)]
 
 
+class QkvProj(ctypes.Structure):
+    """``we_qkv_proj`` of include/we_attn.h."""
+    _fields_ = [("x", c_void_p), ("x_strides", ctypes.c_int64 * 2), ("w", c_void_p), ("w_row_stride", c_int64),
+                ("d_model", c_int32), ("v_out", c_void_p), ("v_out_strides", ctypes.c_int64 * 3)]
+
+
 # name -> (restype, argtypes); must list every symbol include/we_attn.h declares
 SIGNATURES = {
     "we_version": (c_int32, []),
@@ -88,6 +94,28 @@ SIGNATURES = {
         c_int32, c_int32, c_int32, c_int32, c_int32, c_int64,   # B H Hkv T Dh L
         c_int32, c_int32, c_float, c_int32, c_int32, c_int32,  # dilation frozen scale n_splits q_tile dtype
         c_void_p, c_void_p,                        # extras (we_attn_extras* or NULL), stream
+    ]),
+    "we_qkv_rope_kv_store": (c_int32, [
+        c_void_p, c_void_p,                        # proj (we_qkv_proj*), q_out
+        c_void_p, c_void_p, c_int64,               # cos, sin, table_rows
+        c_void_p, c_void_p, c_void_p,              # t_pos, y_pos, x_pos
+        c_int64, c_int64, c_int64,                 # pos_stride_b, grid_h, grid_w
+        c_void_p, c_void_p,                        # kv, written
+        c_int32, c_int32, c_int32, c_int32, c_int32, c_int64,   # B H Hkv T Dh L
+        c_int32, c_int32, c_int32,                 # dilation, is_frozen, dtype
+        c_void_p, c_void_p,                        # extras, stream
+    ]),
+    "we_qkv_rope_kv_attn_fwd": (c_int32, [
+        c_void_p, c_void_p,                        # proj (we_qkv_proj*), q_out
+        c_void_p, c_void_p, c_int64,               # cos, sin, table_rows
+        c_void_p, c_void_p, c_void_p,              # t_pos, y_pos, x_pos
+        c_int64, c_int64, c_int64,                 # pos_stride_b, grid_h, grid_w
+        c_void_p, c_void_p,                        # kv, written
+        c_void_p, _I64x3,                          # out, out_strides
+        c_void_p, c_size_t,                        # workspace, bytes
+        c_int32, c_int32, c_int32, c_int32, c_int32, c_int64,   # B H Hkv T Dh L
+        c_int32, c_int32, c_float, c_int32, c_int32, c_int32,  # dilation frozen scale n_splits q_tile dtype
+        c_void_p, c_void_p,                        # extras, stream
     ]),
 }
 

@@ -14,6 +14,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "_obj")
 # (source, extra defines, object name)
 UNITS = [("rope_kv_store.hip", [], "rope_kv_store.o"),
+         ("qkv_proj_store.hip", [], "qkv_proj_store.o"),
          ("attn_ring.hip", ["-DWE_RING_PART=0"], "attn_ring_bf16_128.o"),
          ("attn_ring.hip", ["-DWE_RING_PART=1"], "attn_ring_bf16_64.o"),
          ("attn_ring.hip", ["-DWE_RING_PART=2"], "attn_ring_f16_128.o"),

@@ -58,6 +58,25 @@ __device__ __forceinline__ void half_wave_pair(float x, float& lower, float& upp
 
 typedef __attribute__((address_space(3))) s16x4_t* lds_s16x4_ptr;
 
+// One 1-KB LDS-DMA: lane i copies 16 bytes from gbase + voff to LDS byte lds_addr + 16*i.
+// Hidden from the compiler's counter bookkeeping on purpose; completion is awaited with
+// dma_wait<N>() (vmcnt) followed by a workgroup barrier.
+__device__ __forceinline__ void dma16(uint64_t gbase, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :
+               : "v"(voff), "s"(gbase), "s"(lds_addr)
+               : "memory", "m0");
+}
+template <int N>
+__device__ __forceinline__ void dma_wait() {
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+__device__ __forceinline__ uint64_t uniform64(uint64_t x) {
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)x);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(x >> 32));
+  return ((uint64_t)hi << 32) | lo;
+}
+
 // Head gate of output row (b, h, t): the given value, or sigmoid(gate_proj(x[b, t, :H]))[h] with
 // the module's rounding steps (src/model/attn.py:117-118: the projection's output and the sigmoid's
 // are both element-type tensors).  The dot product runs in fp32 in channel order.

@@ -72,25 +72,6 @@ __device__ __forceinline__ int v_swz(int row) {
   return DH == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2);
 }
 
-// One 1-KB LDS-DMA: lane i copies 16 bytes from gbase + voff to LDS byte lds_addr + 16*i.
-// Hidden from the compiler's counter bookkeeping on purpose; completion is awaited with
-// dma_wait<N>() (vmcnt) followed by a workgroup barrier.
-__device__ __forceinline__ void dma16(uint64_t gbase, uint32_t voff, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-               :
-               : "v"(voff), "s"(gbase), "s"(lds_addr)
-               : "memory", "m0");
-}
-template <int N>
-__device__ __forceinline__ void dma_wait() {
-  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
-}
-__device__ __forceinline__ uint64_t uniform64(uint64_t x) {
-  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)x);
-  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(x >> 32));
-  return ((uint64_t)hi << 32) | lo;
-}
-
 template <int V>
 struct IntC {
   static constexpr int value = V;

@@ -203,6 +203,80 @@ int prepare_attn(const void* q, const int64_t* q_strides, const void* kv, const 
   return WE_OK;
 }
 
+// Validation of the projection operands and the parameters of the fused projection + store kernel.
+int prepare_proj(const we_qkv_proj* proj, void* q_out, const float* cos_table, const float* sin_table,
+                 int64_t table_rows, const int64_t* t_pos, const int64_t* y_pos, const int64_t* x_pos,
+                 int64_t pos_stride_b, int64_t grid_h, int64_t grid_w, void* kv, uint8_t* written, int B, int H,
+                 int Hkv, int T, int Dh, int64_t L, int dilation, int is_frozen, int dtype,
+                 const we_attn_extras* extras, we::ProjParams& pp) {
+  if (!proj || !proj->x || !proj->w || !q_out || !cos_table || !sin_table || !y_pos || !x_pos || !t_pos || !kv ||
+      !written)
+    return WE_ERR_NULL_POINTER;
+  if (dtype != WE_DTYPE_BF16 && dtype != WE_DTYPE_F16) return WE_ERR_UNSUPPORTED;
+  int rc = ring_shape_ok(B, H, Hkv, T, Dh, L, dilation);
+  if (rc != WE_OK) return rc;
+  if (proj->d_model <= 0 || table_rows <= 0 || grid_h <= 0 || grid_w <= 0) return WE_ERR_BAD_SHAPE;
+  const int64_t feats = (int64_t)(H + 2 * Hkv) * Dh;
+  if ((Dh != 64 && Dh != 128) || proj->d_model % 128 != 0 || feats % 128 != 0 || feats / 128 > (1 << 20))
+    return WE_ERR_UNSUPPORTED;
+  if (proj->w_row_stride < proj->d_model || proj->x_strides[1] < proj->d_model) return WE_ERR_BAD_SHAPE;
+  // per-lane DMA offsets are 32-bit: a frame of x and a 128-row slab of w stay below 2 GiB
+  if ((uint64_t)T * (uint64_t)proj->x_strides[1] * 2u >= (1ull << 31) ||
+      128ull * (uint64_t)proj->w_row_stride * 2u >= (1ull << 31))
+    return WE_ERR_UNSUPPORTED;
+  const int64_t m_tiles = (T + 63) / 64;
+  if (m_tiles * B * 8 * ((feats / 128 + 7) / 8) >= (1ll << 31)) return WE_ERR_UNSUPPORTED;
+  if (!aligned16(proj->x) || !aligned16(proj->w) || !aligned16(q_out) || !aligned16(kv) || !aligned16(cos_table) ||
+      !aligned16(sin_table) || proj->x_strides[0] % 8 != 0 || proj->x_strides[1] % 8 != 0 || proj->w_row_stride % 8 != 0)
+    return WE_ERR_ALIGNMENT;
+  if (proj->v_out && (!aligned16(proj->v_out) || !strides_ok(proj->v_out_strides, dtype))) return WE_ERR_ALIGNMENT;
+
+  we::StoreParams& p = pp.s;
+  p = we::StoreParams{};
+  p.q_out = q_out; p.kv = kv; p.written = written;
+  p.cos_t = cos_table; p.sin_t = sin_table;
+  p.t_pos = t_pos; p.y_pos = y_pos; p.x_pos = x_pos;
+  p.pos_stride_b = pos_stride_b;
+  p.table_rows = table_rows;
+  p.grid_hw = grid_h * grid_w; p.grid_w = grid_w;
+  p.cpr_shift = Dh == 128 ? 3 : 2;
+  p.L = L;
+  p.B = B; p.H = H; p.Hkv = Hkv; p.T = T; p.Dh = Dh;
+  p.dilation = dilation; p.num_buckets = (int)((L / T) / dilation); p.frozen = is_frozen ? 1 : 0;
+  if (extras) {
+    const we_attn_extras& x = *extras;
+    if (x.qk_norm_eps < 0.f || x.qk_norm_eps != x.qk_norm_eps) return WE_ERR_BAD_SHAPE;
+    if ((x.v1 == nullptr) != (x.v_lamb == nullptr)) return WE_ERR_NULL_POINTER;
+    if (x.v1 && (!aligned16(x.v1) || !strides_ok(x.v1_strides, dtype))) return WE_ERR_ALIGNMENT;
+    p.norm_eps = x.qk_norm_eps;
+    p.v1 = x.v1; p.v_lamb = x.v_lamb;
+    p.v1s_b = x.v1_strides[0]; p.v1s_h = x.v1_strides[1]; p.v1s_t = x.v1_strides[2];
+  }
+  pp.x = proj->x; pp.xs_b = proj->x_strides[0]; pp.xs_t = proj->x_strides[1];
+  pp.w = proj->w; pp.ws_n = proj->w_row_stride;
+  pp.K = proj->d_model;
+  pp.v_out = proj->v_out;
+  pp.vo_b = proj->v_out ? proj->v_out_strides[0] : 0;
+  pp.vo_h = proj->v_out ? proj->v_out_strides[1] : 0;
+  pp.vo_t = proj->v_out ? proj->v_out_strides[2] : 0;
+  pp.m_tiles = (int)m_tiles;
+  pp.n_tiles = (int)(feats / 128);
+  return WE_OK;
+}
+
+// the attention module's gate arguments of `extras`
+int apply_gate_extras(const we_attn_extras* extras, int dtype, we::AttnParams& p) {
+  if (!extras) return WE_OK;
+  const we_attn_extras& x = *extras;
+  if ((x.gate_x == nullptr) != (x.gate_w == nullptr)) return WE_ERR_NULL_POINTER;
+  if (x.gate_w != nullptr && (x.gate != nullptr || dtype == WE_DTYPE_F32)) return WE_ERR_UNSUPPORTED;
+  p.gate = x.gate;
+  p.gs_b = x.gate_strides[0]; p.gs_h = x.gate_strides[1]; p.gs_t = x.gate_strides[2];
+  p.gate_x = x.gate_x; p.gate_w = x.gate_w;
+  p.gx_b = x.gate_x_strides[0]; p.gx_t = x.gate_x_strides[1];
+  return WE_OK;
+}
+
 int launch_attn(const we::AttnParams& p, const AttnPlan& pl, int Dh, int dtype, hipStream_t st) {
   if (dtype == WE_DTYPE_F32) return we::launch_attn_ring_f32(p, Dh, st) == hipSuccess ? WE_OK : WE_ERR_LAUNCH;
   const int ksplit = pl.variant == 1 ? 2 : 1;
@@ -380,16 +454,48 @@ int we_rope_kv_attn_fwd(const void* q, const void* k, const void* v, const int64
     sp.norm_eps = x.qk_norm_eps;
     sp.v1 = x.v1; sp.v_lamb = x.v_lamb;
     sp.v1s_b = x.v1_strides[0]; sp.v1s_h = x.v1_strides[1]; sp.v1s_t = x.v1_strides[2];
-    if ((x.gate_x == nullptr) != (x.gate_w == nullptr)) return WE_ERR_NULL_POINTER;
-    if (x.gate_w != nullptr && (x.gate != nullptr || dtype == WE_DTYPE_F32)) return WE_ERR_UNSUPPORTED;
-    p.gate = x.gate;
-    p.gs_b = x.gate_strides[0]; p.gs_h = x.gate_strides[1]; p.gs_t = x.gate_strides[2];
-    p.gate_x = x.gate_x; p.gate_w = x.gate_w;
-    p.gx_b = x.gate_x_strides[0]; p.gx_t = x.gate_x_strides[1];
+    rc = apply_gate_extras(extras, dtype, p);
+    if (rc != WE_OK) return rc;
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
   // Everything is validated before the first launch; the kernels follow each other on the stream.
   if (we::launch_rope_kv_store(sp, dtype, st) != hipSuccess) return WE_ERR_LAUNCH;
+  return launch_attn(p, pl, Dh, dtype, st);
+}
+
+int we_qkv_rope_kv_store(const we_qkv_proj* proj, void* q_out, const float* cos_table, const float* sin_table,
+                         int64_t table_rows, const int64_t* t_pos, const int64_t* y_pos, const int64_t* x_pos,
+                         int64_t pos_stride_b, int64_t grid_h, int64_t grid_w, void* kv, uint8_t* written, int32_t B,
+                         int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L, int32_t dilation,
+                         int32_t is_frozen, int32_t dtype, const we_attn_extras* extras, void* stream) {
+  we::ProjParams pp;
+  const int rc = prepare_proj(proj, q_out, cos_table, sin_table, table_rows, t_pos, y_pos, x_pos, pos_stride_b, grid_h,
+                              grid_w, kv, written, B, H, Hkv, T, Dh, L, dilation, is_frozen, dtype, extras, pp);
+  if (rc != WE_OK) return rc;
+  return we::launch_qkv_rope_store(pp, dtype, static_cast<hipStream_t>(stream)) == hipSuccess ? WE_OK : WE_ERR_LAUNCH;
+}
+
+int we_qkv_rope_kv_attn_fwd(const we_qkv_proj* proj, void* q_out, const float* cos_table, const float* sin_table,
+                            int64_t table_rows, const int64_t* t_pos, const int64_t* y_pos, const int64_t* x_pos,
+                            int64_t pos_stride_b, int64_t grid_h, int64_t grid_w, void* kv, uint8_t* written,
+                            void* out, const int64_t out_strides[3], void* workspace, size_t workspace_bytes,
+                            int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L, int32_t dilation,
+                            int32_t is_frozen, float scale, int32_t n_splits, int32_t q_tile, int32_t dtype,
+                            const we_attn_extras* extras, void* stream) {
+  we::ProjParams pp;
+  int rc = prepare_proj(proj, q_out, cos_table, sin_table, table_rows, t_pos, y_pos, x_pos, pos_stride_b, grid_h,
+                        grid_w, kv, written, B, H, Hkv, T, Dh, L, dilation, is_frozen, dtype, extras, pp);
+  if (rc != WE_OK) return rc;
+  const int64_t qo_strides[3] = {(int64_t)H * T * Dh, (int64_t)T * Dh, (int64_t)Dh};
+  we::AttnParams p;
+  AttnPlan pl;
+  rc = prepare_attn(q_out, qo_strides, kv, written, t_pos, out, out_strides, workspace, workspace_bytes, B, H, Hkv,
+                    T, Dh, L, dilation, scale, n_splits, q_tile, dtype, p, pl);
+  if (rc != WE_OK) return rc;
+  rc = apply_gate_extras(extras, dtype, p);
+  if (rc != WE_OK) return rc;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (we::launch_qkv_rope_store(pp, dtype, st) != hipSuccess) return WE_ERR_LAUNCH;
   return launch_attn(p, pl, Dh, dtype, st);
 }
 

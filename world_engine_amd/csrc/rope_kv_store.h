@@ -133,14 +133,6 @@ __device__ __forceinline__ void rotate_values(const Chunk16<Tag>& in, const floa
     hi.e[i] = Tag::from_f32(y1);
   }
 }
-template <typename Tag>
-__device__ __forceinline__ void rotate_chunk(const Chunk16<Tag>& in, const float* cos_row, const float* sin_row,
-                                             int chunk, Chunk8<Tag>& lo, Chunk8<Tag>& hi) {
-  float c[8], s[8];
-  load_cos_sin(cos_row, sin_row, chunk, c, s);
-  rotate_values<Tag>(in, c, s, lo, hi);
-}
-
 // Destination rows of a K/V item: tail always, ring slot on an unfrozen persisting frame.
 template <typename Tag>
 __device__ __forceinline__ void store_kv_rows(const StoreParams& p, int which, int b, int h, int t, int chunk,
@@ -170,9 +162,72 @@ __device__ __forceinline__ void store_kv_rows(const StoreParams& p, int which, i
   if (!p.frozen && which == 1 && b == 0 && h == 0 && chunk == 0) p.written[to_ring ? ring_row : tail_row] = 1;
 }
 
-// One K (which = 1) or V (which = 2) item: rotate K, copy V; write the tail row always and the
-// ring-slot row when this is an unfrozen persisting frame; mark `written`
-// (src/model/kv_cache.py:138,147-151).
+// Everything after the load of a K (which = 1) or V (which = 2) item: K is normalised (optional)
+// and rotated, V is blended with the value residual (optional); the tail row is written always
+// and the ring-slot row when this is an unfrozen persisting frame; `written` is marked
+// (src/model/attn.py:105-110, src/model/kv_cache.py:138,147-151).  cos / sin are the item's 8
+// table values (used when `rotate`), `res` the matching 16 elements of the value residual (used
+// when p.v1 is set).
+template <typename Tag>
+__device__ __forceinline__ void finish_kv_chunk(const StoreParams& p, int which, int b, int h, int t, int chunk,
+                                                const SlotInfo& si, Chunk16<Tag>& in, bool rotate,
+                                                const float (&c)[8], const float (&s)[8], const Chunk16<Tag>& res,
+                                                float lamb) {
+  if (which == 1 && p.norm_eps > 0.f) rms_norm_chunk<Tag>(in, p.Dh >> 4, p.Dh, p.norm_eps);
+  if (which == 2 && p.v1 != nullptr) lerp_chunk<Tag>(in, res, lamb);
+  Chunk8<Tag> lo, hi;
+  if (rotate) rotate_values<Tag>(in, c, s, lo, hi);
+  store_kv_rows<Tag>(p, which, b, h, t, chunk, si, rotate, in, lo, hi);
+}
+
+// Everything after the load of a Q item: optional norm, rotation (or plain copy when there is no
+// table), store into the contiguous [B, H, T, Dh] output.
+template <typename Tag>
+__device__ __forceinline__ void finish_q_chunk(const StoreParams& p, int b, int h, int t, int chunk,
+                                               Chunk16<Tag>& in, bool rotate, const float (&c)[8],
+                                               const float (&s)[8]) {
+  typedef typename Tag::store_t st_t;
+  if (p.norm_eps > 0.f) rms_norm_chunk<Tag>(in, p.Dh >> 4, p.Dh, p.norm_eps);
+  st_t* dst = (st_t*)p.q_out + (((int64_t)b * p.H + h) * p.T + t) * p.Dh;
+  if (rotate) {
+    Chunk8<Tag> lo, hi;
+    rotate_values<Tag>(in, c, s, lo, hi);
+    store8<Tag>(dst + chunk * 8, lo);
+    store8<Tag>(dst + (p.Dh >> 1) + chunk * 8, hi);
+  } else {
+    store16<Tag>(dst + chunk * 16, in);
+  }
+}
+
+// What an item needs besides its own 16 elements: the 8 cos / sin values of its pairs (rotated
+// items) and the value residual's 16 elements with the blend weight (V items of a layer that has
+// one).  Separate from the arithmetic so that a caller can request them long before it has the
+// item's own values.
+template <typename Tag>
+struct ItemSide {
+  float c[8], s[8];
+  Chunk16<Tag> res;
+  float lamb;
+  bool rotate;
+};
+template <typename Tag>
+__device__ __forceinline__ void load_item_side(const StoreParams& p, int which, int b, int h, int t, int chunk,
+                                               ItemSide<Tag>& sd) {
+  typedef typename Tag::store_t st_t;
+  sd.rotate = which != 2 && p.cos_t != nullptr;
+  sd.lamb = 0.f;
+  if (sd.rotate) {
+    const int64_t pos = rope_table_row(p, b, t);
+    const int half = p.Dh >> 1;
+    load_cos_sin(p.cos_t + pos * half, p.sin_t + pos * half, chunk, sd.c, sd.s);
+  }
+  if (which == 2 && p.v1 != nullptr) {
+    load16<Tag>(sd.res, (const st_t*)p.v1 + b * p.v1s_b + h * p.v1s_h + t * p.v1s_t + chunk * 16);
+    sd.lamb = Tag::to_f32(*reinterpret_cast<const st_t*>(p.v_lamb));
+  }
+}
+
+// One K or V item of the stand-alone store kernel: load, then the above.
 template <typename Tag>
 __device__ __forceinline__ void store_kv_item(const StoreParams& p, int which, int b, int h, int t, int chunk,
                                               const SlotInfo& si) {
@@ -181,20 +236,9 @@ __device__ __forceinline__ void store_kv_item(const StoreParams& p, int which, i
                                : (const st_t*)p.v + b * p.vs_b + h * p.vs_h + t * p.vs_t;
   Chunk16<Tag> in;
   load16<Tag>(in, src + chunk * 16);
-  if (which == 1 && p.norm_eps > 0.f) rms_norm_chunk<Tag>(in, p.Dh >> 4, p.Dh, p.norm_eps);
-  if (which == 2 && p.v1 != nullptr) {
-    Chunk16<Tag> res;
-    load16<Tag>(res, (const st_t*)p.v1 + b * p.v1s_b + h * p.v1s_h + t * p.v1s_t + chunk * 16);
-    lerp_chunk<Tag>(in, res, Tag::to_f32(*reinterpret_cast<const st_t*>(p.v_lamb)));
-  }
-  const bool rotate = which == 1 && p.cos_t != nullptr;
-  Chunk8<Tag> lo, hi;
-  if (rotate) {
-    const int64_t pos = rope_table_row(p, b, t);
-    const int half = p.Dh >> 1;
-    rotate_chunk<Tag>(in, p.cos_t + pos * half, p.sin_t + pos * half, chunk, lo, hi);
-  }
-  store_kv_rows<Tag>(p, which, b, h, t, chunk, si, rotate, in, lo, hi);
+  ItemSide<Tag> sd;
+  load_item_side<Tag>(p, which, b, h, t, chunk, sd);
+  finish_kv_chunk<Tag>(p, which, b, h, t, chunk, si, in, sd.rotate, sd.c, sd.s, sd.res, sd.lamb);
 }
 
 }  // namespace we

@@ -42,18 +42,9 @@ __global__ void __launch_bounds__(256) rope_kv_store_kernel(StoreParams p) {
   const int h = head_all;
   Chunk16<Tag> in;
   load16<Tag>(in, (const st_t*)p.q + b * p.qs_b + h * p.qs_h + t * p.qs_t + chunk * 16);
-  if (p.norm_eps > 0.f) rms_norm_chunk<Tag>(in, cpr, p.Dh, p.norm_eps);
-  st_t* dst = (st_t*)p.q_out + (((int64_t)b * p.H + h) * p.T + t) * p.Dh;
-  if (p.cos_t != nullptr) {
-    const int64_t pos = rope_table_row(p, b, t);
-    const int half = p.Dh >> 1;
-    Chunk8<Tag> lo, hi;
-    rotate_chunk<Tag>(in, p.cos_t + pos * half, p.sin_t + pos * half, chunk, lo, hi);
-    store8<Tag>(dst + chunk * 8, lo);
-    store8<Tag>(dst + half + chunk * 8, hi);
-  } else {
-    store16<Tag>(dst + chunk * 16, in);
-  }
+  ItemSide<Tag> sd;
+  load_item_side<Tag>(p, 0, b, h, t, chunk, sd);
+  finish_q_chunk<Tag>(p, b, h, t, chunk, in, sd.rotate, sd.c, sd.s);
 }
 
 hipError_t launch_rope_kv_store(const StoreParams& p, int dtype, hipStream_t stream) {

@@ -68,7 +68,22 @@ struct AttnParams {
   uint64_t* clock_out;
 };
 
+// The merged q/k/v projection with the store's work as its epilogue (qkv_proj_store.hip).
+struct ProjParams {
+  StoreParams s;        // q / k / v inputs unused; everything else as for the store kernel
+  const void* x;        // [B, T, K] module input, channel stride 1
+  int64_t xs_b, xs_t;   // element strides
+  const void* w;        // [(H + 2 Hkv) Dh, K] merged projection weight, row-major (out, in)
+  int64_t ws_n;         // element stride between weight rows
+  int K;                // d_model
+  void* v_out;          // optional: the projected v rows before the blend (the layer's v1 output)
+  int64_t vo_b, vo_h, vo_t;
+  int m_tiles;          // ceil(T / 64)
+  int n_tiles;          // (H + 2 Hkv) Dh / 128
+};
+
 hipError_t launch_rope_kv_store(const StoreParams& p, int dtype, hipStream_t stream);
+hipError_t launch_qkv_rope_store(const ProjParams& p, int dtype, hipStream_t stream);
 
 // main kernel, one launcher per (element type, head dim) family: ksplit = 2 -> 128 queries per
 // workgroup, 1 -> 256

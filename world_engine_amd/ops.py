@@ -258,6 +258,39 @@ def attn_ring_static(q: Tensor, kv: Tensor, written: Tensor, t_pos: Tensor, L: i
     return out
 
 
+def _build_extras(dtype, B, H, Hkv, T, Dh, qk_norm_eps, v1, v_lamb, gate, gate_x, gate_w):
+    """``we_attn_extras`` for a call, or None.  Returns (pointer or None, object to keep alive)."""
+    if not (qk_norm_eps or v1 is not None or gate is not None or gate_w is not None):
+        return None, None
+    ex = _capi.AttnExtras()
+    ex.qk_norm_eps = float(qk_norm_eps)
+    if v1 is not None:
+        if (v_lamb is None or v_lamb.numel() != 1 or v_lamb.dtype != dtype or tuple(v1.shape) != (B, Hkv, T, Dh)
+                or v1.dtype != dtype):
+            raise RuntimeError("v1 must match v and v_lamb must be one element of the same type")
+        _need_device(v1, v_lamb)
+        ex.v1, ex.v_lamb = v1.data_ptr(), v_lamb.data_ptr()
+        ex.v1_strides = _bhtd_strides(v1, "v1")
+    if gate is not None:
+        if tuple(gate.shape) != (B, H, T) or gate.dtype != dtype:
+            raise RuntimeError("gate must be [B, H, T] of q's element type")
+        _need_device(gate)
+        ex.gate = gate.data_ptr()
+        ex.gate_strides = _capi.i64x3(*gate.stride())
+    if gate_w is not None:
+        if gate is not None:
+            raise RuntimeError("give either gate or gate_x / gate_w")
+        if (gate_x is None or gate_x.dim() != 3 or tuple(gate_x.shape) != (B, T, H) or gate_x.stride(2) != 1
+                or gate_x.dtype != dtype or tuple(gate_w.shape) != (H, H) or gate_w.dtype != dtype
+                or not gate_w.is_contiguous()):
+            raise RuntimeError("gate_x must be [B, T, H] (contiguous channels) and gate_w a contiguous [H, H], "
+                               "both of q's element type")
+        _need_device(gate_x, gate_w)
+        ex.gate_x, ex.gate_w = gate_x.data_ptr(), gate_w.data_ptr()
+        ex.gate_x_strides = (ctypes.c_int64 * 2)(gate_x.stride(0), gate_x.stride(1))
+    return ctypes.byref(ex), ex
+
+
 def rope_kv_attn(q: Tensor, k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor], cos_table: Tensor,
                  sin_table: Tensor, grid_h: int, grid_w: int, kv: Tensor, written: Tensor, L: int,
                  dilation: int, is_frozen: bool, scale: Optional[float] = None, n_splits: int = 0,
@@ -301,34 +334,7 @@ def rope_kv_attn(q: Tensor, k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor],
             out = torch.empty((B, H, T, Dh), dtype=q.dtype, device=dev)
     elif tuple(out.shape) != (B, H, T, Dh) or out.dtype != q.dtype or out.device != dev:
         raise RuntimeError("out must be [B, H, T, Dh] of q's element type on q's device")
-    extras = None
-    if qk_norm_eps or v1 is not None or gate is not None or gate_w is not None:
-        ex = _capi.AttnExtras()
-        ex.qk_norm_eps = float(qk_norm_eps)
-        if v1 is not None:
-            if v_lamb is None or v_lamb.numel() != 1 or v_lamb.dtype != v.dtype or v1.shape != v.shape or v1.dtype != v.dtype:
-                raise RuntimeError("v1 must match v and v_lamb must be one element of the same type")
-            _need_device(v1, v_lamb)
-            ex.v1, ex.v_lamb = v1.data_ptr(), v_lamb.data_ptr()
-            ex.v1_strides = _bhtd_strides(v1, "v1")
-        if gate is not None:
-            if tuple(gate.shape) != (B, H, T) or gate.dtype != q.dtype:
-                raise RuntimeError("gate must be [B, H, T] of q's element type")
-            _need_device(gate)
-            ex.gate = gate.data_ptr()
-            ex.gate_strides = _capi.i64x3(*gate.stride())
-        if gate_w is not None:
-            if gate is not None:
-                raise RuntimeError("give either gate or gate_x / gate_w")
-            if (gate_x is None or gate_x.dim() != 3 or tuple(gate_x.shape) != (B, T, H) or gate_x.stride(2) != 1
-                    or gate_x.dtype != q.dtype or tuple(gate_w.shape) != (H, H) or gate_w.dtype != q.dtype
-                    or not gate_w.is_contiguous()):
-                raise RuntimeError("gate_x must be [B, T, H] (contiguous channels) and gate_w a contiguous [H, H], "
-                                   "both of q's element type")
-            _need_device(gate_x, gate_w)
-            ex.gate_x, ex.gate_w = gate_x.data_ptr(), gate_w.data_ptr()
-            ex.gate_x_strides = (ctypes.c_int64 * 2)(gate_x.stride(0), gate_x.stride(1))
-        extras = ctypes.byref(ex)
+    extras, _keep = _build_extras(q.dtype, B, H, Hkv, T, Dh, qk_norm_eps, v1, v_lamb, gate, gate_x, gate_w)
     code = _call(
         dev, lib.we_rope_kv_attn_fwd,
         q.data_ptr(), k.data_ptr(), v.data_ptr(), _bhtd_strides(q, "q"), _bhtd_strides(k, "k"), _bhtd_strides(v, "v"),
@@ -341,6 +347,71 @@ def rope_kv_attn(q: Tensor, k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor],
         extras, _stream_ptr(dev))
     _capi.check(code, "we_rope_kv_attn_fwd")
     return out, q_rot
+
+
+def qkv_rope_kv_attn(x: Tensor, w_qkv: Tensor, n_heads: int, n_kv_heads: int, pos_ids: Mapping[str, Tensor],
+                     cos_table: Tensor, sin_table: Tensor, grid_h: int, grid_w: int, kv: Tensor, written: Tensor,
+                     L: int, dilation: int, is_frozen: bool, scale: Optional[float] = None, n_splits: int = 0,
+                     q_tile: int = 0, attend: bool = True, want_v: bool = False, qk_norm_eps: float = 0.0,
+                     v1: Optional[Tensor] = None, v_lamb: Optional[Tensor] = None, gate: Optional[Tensor] = None,
+                     gate_x: Optional[Tensor] = None, gate_w: Optional[Tensor] = None):
+    """The module's merged q/k/v projection, RoPE, the cache write and (``attend``) the attention
+    over the ring in one library call (``we_qkv_rope_kv_attn_fwd`` / ``we_qkv_rope_kv_store``):
+    ``src/patch_model.py:116-134`` from ``self.qkv_proj(x)`` to the ``flex_attention`` call.  The
+    projection runs in the library's own kernel with the store's work as its epilogue, so q, k, v
+    never exist as a ``[B, T, (H + 2 Hkv) Dh]`` tensor.
+
+    ``x`` ``[B, T, d_model]`` (channel stride 1), ``w_qkv`` ``[(H + 2 Hkv) Dh, d_model]`` =
+    ``qkv_proj.weight``.  Returns ``(out or None, q_rot, v or None)``: ``out`` ``[B, H, T, Dh]`` in
+    token-major memory, ``q_rot`` the rotated (normalised) queries, ``v`` (``want_v``) the projected
+    value rows ``[B, Hkv, T, Dh]`` before the value blend - what the first layer returns as ``v1``.
+    Projection rows are fp32 sums rounded once to the element type in a fixed order that differs
+    from a BLAS library's: they can differ from ``F.linear``'s in the last bit."""
+    dev = _need_device(x, w_qkv, kv, written, cos_table, sin_table, pos_ids["t_pos"])
+    if x.dim() != 3 or x.stride(2) != 1:
+        raise RuntimeError("x must be [B, T, d_model] with contiguous channels")
+    B, T, d_model = x.shape
+    if kv.dim() != 5:
+        raise RuntimeError("kv must be [2, B, Hkv, L+T, Dh]")
+    Dh = kv.shape[4]
+    H, Hkv = n_heads, n_kv_heads
+    if w_qkv.dim() != 2 or tuple(w_qkv.shape) != ((H + 2 * Hkv) * Dh, d_model) or w_qkv.stride(1) != 1:
+        raise RuntimeError("w_qkv must be [(H + 2 Hkv) * Dh, d_model] with contiguous rows")
+    if x.dtype != kv.dtype or w_qkv.dtype != kv.dtype:
+        raise RuntimeError("x and w_qkv must have the cache's element type")
+    _check_cache(kv, written, B, Hkv, T, Dh, L)
+    _check_tables(cos_table, sin_table, Dh)
+    t_pos, y_pos, x_pos, ps = _pos_triplet(pos_ids, B, T, True)
+    scale = 1.0 / math.sqrt(Dh) if scale is None else float(scale)
+    lib = _capi.lib()
+    q_rot = torch.empty((B, H, T, Dh), dtype=x.dtype, device=dev)
+    proj = _capi.QkvProj()
+    proj.x, proj.w, proj.d_model = x.data_ptr(), w_qkv.data_ptr(), d_model
+    proj.x_strides = (ctypes.c_int64 * 2)(x.stride(0), x.stride(1))
+    proj.w_row_stride = w_qkv.stride(0)
+    v_raw = None
+    if want_v:   # token-major like the projection output the module would have sliced it from
+        v_raw = torch.empty((B, T, Hkv, Dh), dtype=x.dtype, device=dev).transpose(1, 2)
+        proj.v_out = v_raw.data_ptr()
+        proj.v_out_strides = _bhtd_strides(v_raw, "v_out")
+    extras, _keep = _build_extras(x.dtype, B, H, Hkv, T, Dh, qk_norm_eps, v1, v_lamb, gate, gate_x, gate_w)
+    head = (ctypes.byref(proj), q_rot.data_ptr(), cos_table.data_ptr(), sin_table.data_ptr(), cos_table.shape[0],
+            t_pos.data_ptr(), y_pos.data_ptr(), x_pos.data_ptr(), ps, grid_h, grid_w, kv.data_ptr(),
+            written.data_ptr())
+    if not attend:
+        code = _call(dev, lib.we_qkv_rope_kv_store, *head, B, H, Hkv, T, Dh, L, dilation, int(bool(is_frozen)),
+                     _dtype_code(kv), extras, _stream_ptr(dev))
+        _capi.check(code, "we_qkv_rope_kv_store")
+        return None, q_rot, v_raw
+    ws_bytes = int(lib.we_attn_workspace_bytes(B, H, Hkv, T, Dh, L, n_splits, q_tile))
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+    out = torch.empty((B, T, H, Dh), dtype=x.dtype, device=dev).transpose(1, 2)
+    code = _call(dev, lib.we_qkv_rope_kv_attn_fwd, *head, out.data_ptr(), _bhtd_strides(out, "out"),
+                 workspace.data_ptr() if ws_bytes else None, ws_bytes,
+                 B, H, Hkv, T, Dh, L, dilation, int(bool(is_frozen)), scale, n_splits, q_tile, _dtype_code(kv),
+                 extras, _stream_ptr(dev))
+    _capi.check(code, "we_qkv_rope_kv_attn_fwd")
+    return out, q_rot, v_raw
 
 
 # --------------------------------------------------------------------------------------------
@@ -393,3 +464,26 @@ def _rope_kv_attn_fake(q, k, v, t_pos, y_pos, x_pos, cos_table, sin_table, grid_
                        gate_w=None):
     B, H, T, Dh = q.shape
     return q.new_empty((B, T, H, Dh)).transpose(1, 2)
+
+
+@torch.library.custom_op("world_engine_amd::qkv_rope_kv_attn", mutates_args=("kv", "written"))
+def qkv_rope_kv_attn_op(x: Tensor, w_qkv: Tensor, n_heads: int, n_kv_heads: int, t_pos: Tensor, y_pos: Tensor,
+                        x_pos: Tensor, cos_table: Tensor, sin_table: Tensor, grid_h: int, grid_w: int,
+                        kv: Tensor, written: Tensor, L: int, dilation: int, is_frozen: bool, scale: float,
+                        qk_norm_eps: float = 0.0, v1: Optional[Tensor] = None, v_lamb: Optional[Tensor] = None,
+                        gate_x: Optional[Tensor] = None, gate_w: Optional[Tensor] = None) -> Tuple[Tensor, Tensor]:
+    """Returns (attention output, projected v rows before the value blend)."""
+    pos = {"t_pos": t_pos, "y_pos": y_pos, "x_pos": x_pos}
+    out, _, v = qkv_rope_kv_attn(x, w_qkv, n_heads, n_kv_heads, pos, cos_table, sin_table, grid_h, grid_w, kv,
+                                 written, L, dilation, is_frozen, scale, want_v=True, qk_norm_eps=qk_norm_eps,
+                                 v1=v1, v_lamb=v_lamb, gate_x=gate_x, gate_w=gate_w)
+    return out, v
+
+
+@qkv_rope_kv_attn_op.register_fake
+def _qkv_rope_kv_attn_fake(x, w_qkv, n_heads, n_kv_heads, t_pos, y_pos, x_pos, cos_table, sin_table, grid_h, grid_w,
+                           kv, written, L, dilation, is_frozen, scale, qk_norm_eps=0.0, v1=None, v_lamb=None,
+                           gate_x=None, gate_w=None):
+    B, T = x.shape[:2]
+    Dh = kv.shape[4]
+    return (x.new_empty((B, T, n_heads, Dh)).transpose(1, 2), x.new_empty((B, T, n_kv_heads, Dh)).transpose(1, 2))
