@@ -380,7 +380,8 @@ def run_cpu(cfg_id, c, args, torch, ro, threads=None, dtype=None, budget=None):
 def run_module(args, torch, ro, wea):
     """The attention module around the path at cfg1 shapes (d_model 2048, merged QKV projection,
     value residual and head gate, output projection), 20 layers' worth in one HIP graph: with the
-    element-wise neighbours as torch operations and with them inside the kernels."""
+    element-wise neighbours as torch operations, with them inside the kernels, and with the q/k/v
+    projection inside the library's store kernel as well."""
     from types import SimpleNamespace
     dev = torch.device("cuda:0")
     T, H, Dh, n = 256, 16, 128, 16
@@ -390,9 +391,10 @@ def run_module(args, torch, ro, wea):
     cos, sin = ro.rope_table_1d(64 * T, Dh)
     rope = wea.RoPE(cos, sin, 16, 16).to(dev)
     res = {}
-    for fuse in (False, True):
+    for fuse, fuse_proj in ((False, False), (True, False), (True, True)):
         torch.manual_seed(0)
-        mod = wea.RingAttn(cfg, 0, rope, merged_qkv=True, fuse_elementwise=fuse).to(dev, torch.bfloat16)
+        mod = wea.RingAttn(cfg, 0, rope, merged_qkv=True, fuse_elementwise=fuse,
+                           fuse_projection=fuse_proj).to(dev, torch.bfloat16)
         cache = wea.StaticKVCache(cfg, 1, torch.bfloat16).to(dev)
         cache.set_frozen(False)
         for layer in cache.layers:
@@ -420,7 +422,8 @@ def run_module(args, torch, ro, wea):
                     g.replay()
                 torch.cuda.synchronize()
                 xs.append((time.perf_counter() - t0) / 200 * 1e6)
-        res["fused_elementwise" if fuse else "torch_elementwise"] = round(percentile(xs, 0.5), 2)
+        key = "fused_projection" if fuse_proj else ("fused_elementwise" if fuse else "torch_elementwise")
+        res[key] = round(percentile(xs, 0.5), 2)
         del mod, cache, g
     res["what"] = ("us per RingAttn.forward at cfg1 shapes (d_model 2048, merged qkv_proj, value residual, head gate, "
                    "out_proj included), 20 calls per HIP graph")

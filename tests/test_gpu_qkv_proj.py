@@ -131,3 +131,54 @@ def test_projection_rejects_bad_operands(gpu_device):
     before = lay.kv.clone()
     torch.cuda.synchronize()
     assert torch.equal(before, lay.kv)
+
+
+@pytest.mark.parametrize("compiled", [False, True])
+def test_module_with_fused_projection(gpu_device, compiled):
+    """RingAttn(fuse_projection=True) - x in, out_proj's input out, two library kernels and the
+    combine in between - against the same module with the projection as a torch linear layer, two
+    layers deep so that the first layer's projected v reaches the second as the value residual;
+    also under torch.compile(fullgraph=True), where the call is the registered opaque op."""
+    import types
+    import world_engine_amd as wea
+    torch.manual_seed(2)
+    dev = gpu_device
+    cfg = types.SimpleNamespace(d_model=512, n_heads=4, n_kv_heads=2, value_residual=True, gated_attn=True,
+                                tokens_per_frame=64, local_window=3, global_window=3, global_attn_period=1,
+                                global_pinned_dilation=1, n_layers=2)
+    cos, sin = ro.rope_table_1d(16 * 64, 128)
+    rope = wea.RoPE(cos, sin, 8, 8).to(dev)
+    plain = [wea.RingAttn(cfg, i, rope, merged_qkv=True, fuse_elementwise=True).to(dev, torch.bfloat16)
+             for i in range(2)]
+    fused = [wea.RingAttn(cfg, i, rope, merged_qkv=True, fuse_elementwise=True, fuse_projection=True)
+             .to(dev, torch.bfloat16) for i in range(2)]
+    for a, b in zip(plain, fused):
+        with torch.no_grad():
+            a.gate_proj.weight.normal_(0, 0.5)
+            a.v_lamb.fill_(0.3)
+        b.load_state_dict(a.state_dict())
+    run = [torch.compile(m, fullgraph=True) for m in fused] if compiled else fused
+    caches = [wea.StaticKVCache(cfg, 1, torch.bfloat16).to(dev) for _ in range(2)]
+    for c in caches:
+        c.set_frozen(False)
+        for layer in c.layers:
+            layer.check_inputs = False
+    for t in range(5):
+        print(f"module fused projection compiled={compiled} t={t}", flush=True)
+        x = torch.randn(1, 64, 512, device=dev, dtype=torch.bfloat16)
+        pos = to_dev(ro.synth_pos_ids(t, 1, 64, 8), dev)
+        with torch.no_grad():
+            ya, v1a = plain[0](x, pos, None, caches[0])
+            ya2, _ = plain[1](ya, pos, v1a, caches[0])
+            yb, v1b = run[0](x, pos, None, caches[1])
+            yb2, _ = run[1](yb, pos, v1b, caches[1])
+        assert v1b.shape == v1a.shape
+        assert_ulp_close(v1b, v1a, f"v1 t={t}")
+        d1 = (ya.float() - yb.float()).abs().max().item()
+        d2 = (ya2.float() - yb2.float()).abs().max().item()
+        assert d1 <= 2e-2 * max(1.0, ya.float().abs().max().item()), (t, d1)
+        assert d2 <= 3e-2 * max(1.0, ya2.float().abs().max().item()), (t, d2)
+        for li in range(2):
+            assert_ulp_close(caches[1].layers[li].kv, caches[0].layers[li].kv, f"layer {li} cache t={t}",
+                             ulps=2 if li else 1)
+            assert torch.equal(caches[1].layers[li].written, caches[0].layers[li].written)

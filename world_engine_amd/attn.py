@@ -136,12 +136,20 @@ class RingAttn(nn.Module):
     norm, value-residual lerp, head gate incl. its H x H projection and sigmoid) into the two
     kernels: seven to nine launches fewer per layer, results within 1 ulp of the separate torch operations instead of bit-identical, which
     is why it is off unless asked for.
+
+    ``fuse_projection`` (on top of ``merged_qkv`` and ``fuse_elementwise``) also runs the merged
+    q/k/v projection in the library, in one kernel with the cache write: x goes in, the rotated q
+    and the cache rows come out, the ``[B, T, (H + 2 Hkv) Dh]`` projection output never exists.
+    Its rows are fp32 sums rounded once like the BLAS routine's, in another order of additions.
     """
 
     def __init__(self, config, layer_idx: int, rope: RoPE, merged_qkv: bool = False,
-                 fuse_elementwise: bool = False):
+                 fuse_elementwise: bool = False, fuse_projection: bool = False):
         super().__init__()
+        if fuse_projection and not (merged_qkv and fuse_elementwise):
+            raise AssertionError("fuse_projection needs merged_qkv and fuse_elementwise")
         self.fuse_elementwise = fuse_elementwise
+        self.fuse_projection = fuse_projection
         self.config = config
         self.layer_idx = layer_idx
         self.n_heads = config.n_heads
@@ -174,10 +182,11 @@ class RingAttn(nn.Module):
 
     @classmethod
     def from_reference(cls, src: nn.Module, config, rope: RoPE, merged_qkv: bool = True,
-                       fuse_elementwise: bool = False):
+                       fuse_elementwise: bool = False, fuse_projection: bool = False):
         """Build from an ``Attn``-like module (anything with ``layer_idx`` and a matching state
         dict), the way the reference's ``MergedQKVAttn(src, config)`` does."""
-        new = cls(config, src.layer_idx, rope, merged_qkv=merged_qkv, fuse_elementwise=fuse_elementwise)
+        new = cls(config, src.layer_idx, rope, merged_qkv=merged_qkv, fuse_elementwise=fuse_elementwise,
+                  fuse_projection=fuse_projection)
         ref_w = next(src.parameters())
         new.to(device=ref_w.device, dtype=ref_w.dtype)
         state = {k: v for k, v in src.state_dict().items()}
@@ -188,8 +197,26 @@ class RingAttn(nn.Module):
         new.train(src.training)
         return new
 
+    def _forward_fused_projection(self, x: Tensor, pos_ids, v1: Optional[Tensor], kv_cache):
+        """x -> [projection + norm + RoPE + value blend + cache write] -> [attention + gate] -> out_proj."""
+        B, T = x.shape[:2]
+        extras = {"qk_norm_eps": torch.finfo(torch.float32).eps}
+        first = self.value_residual and v1 is None
+        if self.value_residual and not first:
+            extras.update(v1=v1.view(B, self.n_kv_heads, T, self.d_head), v_lamb=self.v_lamb)
+        if self.gated_attn:
+            extras.update(gate_x=x[..., : self.n_heads], gate_w=self.gate_proj.weight)
+        y, v = kv_cache.qkv_rope_upsert_attend(x, self.qkv_proj.weight, self.n_heads, pos_ids, self.rope,
+                                               self.layer_idx, want_v=first, **extras)
+        if first:
+            v1 = v
+        return self.out_proj(y.transpose(1, 2).reshape(B, T, -1)), v1
+
     def forward(self, x: Tensor, pos_ids: Mapping[str, Tensor], v1: Optional[Tensor], kv_cache):
         B, T = x.shape[:2]
+        if (self.fuse_projection and hasattr(kv_cache, "qkv_rope_upsert_attend")
+                and x.dtype in (torch.bfloat16, torch.float16) and x.stride(-1) == 1):
+            return self._forward_fused_projection(x, pos_ids, v1, kv_cache)
         if self.merged_qkv:
             q, k, v = self.qkv_proj(x).split((self.q_out, self.kv_out, self.kv_out), dim=-1)
         else:
@@ -235,13 +262,14 @@ class RingAttn(nn.Module):
 
 
 def install_ring_attention(model: nn.Module, rope: RoPE, attn_types: tuple, merged_qkv: bool = True,
-                           fuse_elementwise: bool = False) -> int:
+                           fuse_elementwise: bool = False, fuse_projection: bool = False) -> int:
     """Swap every submodule that is an instance of ``attn_types`` for a :class:`RingAttn`, the
     same ``set_submodule`` walk the reference uses for its merged-QKV patch
     (``src/patch_model.py:144-147``).  Returns the number of modules replaced."""
     n = 0
     for name, mod in list(model.named_modules()):
         if isinstance(mod, attn_types) and not isinstance(mod, RingAttn):
-            model.set_submodule(name, RingAttn.from_reference(mod, model.config, rope, merged_qkv, fuse_elementwise))
+            model.set_submodule(name, RingAttn.from_reference(mod, model.config, rope, merged_qkv, fuse_elementwise,
+                                                                 fuse_projection))
             n += 1
     return n

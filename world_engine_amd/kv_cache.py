@@ -135,6 +135,30 @@ class LayerKVCache(nn.Module):
                                 qk_norm_eps=qk_norm_eps, v1=v1, v_lamb=v_lamb, gate=gate, gate_x=gate_x,
                                 gate_w=gate_w)[0]
 
+    def qkv_rope_upsert_attend(self, x: Tensor, w_qkv: Tensor, n_heads: int, pos_ids: Mapping[str, Tensor], rope,
+                               is_frozen: bool, scale: Optional[float] = None, want_v: bool = False,
+                               qk_norm_eps: float = 0.0, v1: Optional[Tensor] = None,
+                               v_lamb: Optional[Tensor] = None, gate_x: Optional[Tensor] = None,
+                               gate_w: Optional[Tensor] = None) -> Tuple[Tensor, Optional[Tensor]]:
+        """``rope_upsert_attend`` with the module's merged q/k/v projection in front, as one
+        library call (``src/patch_model.py:116-134`` from ``self.qkv_proj(x)`` to the attention
+        output).  Returns ``(y, v)``: ``v`` (``want_v``) is the projected value rows before the
+        value blend, what the first layer hands on as ``v1``."""
+        n_kv = self.kv.shape[2]
+        if torch.compiler.is_compiling():
+            s = float(scale) if scale is not None else float(self.kv.shape[4]) ** -0.5
+            y, v = torch.ops.world_engine_amd.qkv_rope_kv_attn(
+                x, w_qkv, n_heads, n_kv, pos_ids["t_pos"], pos_ids["y_pos"], pos_ids["x_pos"], rope.cos, rope.sin,
+                rope.height, rope.width, self.kv, self.written, self.L, self.pinned_dilation, bool(is_frozen), s,
+                float(qk_norm_eps), v1, v_lamb, gate_x, gate_w)
+            return y, (v if want_v else None)
+        self._check(x.unsqueeze(1), pos_ids, rope)
+        y, _, v = ops.qkv_rope_kv_attn(x, w_qkv, n_heads, n_kv, pos_ids, rope.cos, rope.sin, rope.height, rope.width,
+                                       self.kv, self.written, self.L, self.pinned_dilation, is_frozen, scale,
+                                       want_v=want_v, qk_norm_eps=qk_norm_eps, v1=v1, v_lamb=v_lamb, gate_x=gate_x,
+                                       gate_w=gate_w)
+        return y, v
+
 
 class StaticKVCache(nn.Module):
     """Per-layer rings with local/global windows chosen as in ``src/model/kv_cache.py:157-181``."""
@@ -172,3 +196,8 @@ class StaticKVCache(nn.Module):
     def rope_upsert_attend(self, q: Tensor, k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor], rope, layer: int,
                            scale: Optional[float] = None, **extras) -> Tensor:
         return self.layers[layer].rope_upsert_attend(q, k, v, pos_ids, rope, self._is_frozen, scale, **extras)
+
+    def qkv_rope_upsert_attend(self, x: Tensor, w_qkv: Tensor, n_heads: int, pos_ids: Mapping[str, Tensor], rope,
+                               layer: int, scale: Optional[float] = None, **extras):
+        return self.layers[layer].qkv_rope_upsert_attend(x, w_qkv, n_heads, pos_ids, rope, self._is_frozen, scale,
+                                                         **extras)
