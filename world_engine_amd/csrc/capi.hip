@@ -220,7 +220,7 @@ int prepare_proj(const we_qkv_proj* proj, void* q_out, const float* cos_table, c
   if ((Dh != 64 && Dh != 128) || proj->d_model % 128 != 0 || feats % 128 != 0 || feats / 128 > (1 << 20))
     return WE_ERR_UNSUPPORTED;
   if (proj->w_row_stride < proj->d_model || proj->x_strides[1] < proj->d_model) return WE_ERR_BAD_SHAPE;
-  // per-lane DMA offsets are 32-bit: a frame of x and a 128-row slab of w stay below 2 GiB
+  // per-lane offsets are 32-bit: a frame of x and a 128-row slab of w stay below 2 GiB
   if ((uint64_t)T * (uint64_t)proj->x_strides[1] * 2u >= (1ull << 31) ||
       128ull * (uint64_t)proj->w_row_stride * 2u >= (1ull << 31))
     return WE_ERR_UNSUPPORTED;
