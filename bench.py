@@ -430,6 +430,63 @@ def run_module(args, torch, ro, wea):
     return res
 
 
+def run_projection(torch, ro, wea, ops):
+    """The producer side of the path at cfg1's module shapes: the merged q/k/v projection + RoPE + cache
+    write as the library's one kernel (we_qkv_rope_kv_store) against torch's linear layer followed by the
+    store kernel, both over 20 distinct weight matrices per HIP graph (500 MB: every call streams its
+    weights from HBM, as the layers of a model do)."""
+    dev = torch.device("cuda:0")
+    T, H, Dh, n, dm = 256, 16, 128, 16, 2048
+    cos, sin = ro.rope_table_1d(64 * T, Dh)
+    rope = wea.RoPE(cos, sin, 16, 16).to(dev)
+    kv = torch.zeros(2, 1, H, (n + 1) * T, Dh, device=dev, dtype=torch.bfloat16)
+    written = torch.zeros((n + 1) * T, dtype=torch.bool, device=dev)
+    written[n * T:] = True
+    x = torch.randn(1, T, dm, device=dev, dtype=torch.bfloat16)
+    ws = [(torch.randn(3 * H * Dh, dm, device=dev) / dm ** 0.5).to(torch.bfloat16) for _ in range(20)]
+    poss = [{k: v.to(dev) for k, v in ro.synth_pos_ids(t, 1, T, 16).items()} for t in range(40)]
+
+    def fused(t, w):
+        ops.qkv_rope_kv_attn(x, w, H, H, poss[t], rope.cos, rope.sin, 16, 16, kv, written, n * T, 1, False,
+                             attend=False)
+
+    def separate(t, w):
+        q, k, v = torch.nn.functional.linear(x, w).split((H * Dh, H * Dh, H * Dh), dim=-1)
+        q, k, v = (z.reshape(1, T, H, Dh).transpose(1, 2) for z in (q, k, v))
+        ops.rope_kv_store(q, k, v, poss[t], rope.cos, rope.sin, 16, 16, kv, written, n * T, 1, False)
+
+    res = {}
+    for name, fn in (("fused_kernel", fused), ("linear_plus_store_kernel", separate)):
+        for t in range(20):
+            fn(t, ws[t])
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.graph(g, stream=s):
+            for t in range(20, 40):
+                fn(t, ws[t - 20])
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        xs = []
+        for _ in range(SAMPLES):
+            t0 = time.perf_counter()
+            for _ in range(10):
+                g.replay()
+            torch.cuda.synchronize()
+            xs.append((time.perf_counter() - t0) / 200 * 1e6)
+        res[name] = round(percentile(xs, 0.5), 2)
+        del g
+    alg = 2 * dm * 3 * H * Dh + 2 * T * dm + 2 * T * H * Dh * (1 + 2 * 2)   # W + x read; q_out + tail + ring rows written
+    res["algorithmic_bytes"] = alg
+    res["fused_gbps"] = round(alg / res["fused_kernel"] / 1e3, 1)
+    res["fused_frac_of_hbm_peak"] = round(alg / res["fused_kernel"] / 1e3 / 8000.0, 4)
+    res["what"] = ("us per call at cfg1's module shapes (x [1,256,2048], merged weight [6144,2048], 16 heads of 128, persisting "
+                   "frame), 20 distinct weight matrices per HIP graph")
+    return res
+
+
 def run_peaks(torch):
     """What this box reaches on library code, next to the published peaks the roofline is priced
     against: a bf16 GEMM through hipBLASLt and a streaming copy."""
@@ -500,7 +557,8 @@ def main():
 
     torch.cuda.set_device(0)
     if args.module_only:
-        print(json.dumps({"module": run_module(args, torch, ro, wea)}), flush=True)
+        print(json.dumps({"module": run_module(args, torch, ro, wea),
+                          "projection": run_projection(torch, ro, wea, ops)}), flush=True)
         return
     single = args.config != 0
     cfg_ids = [args.config] if single else sorted(CONFIGS)
@@ -529,6 +587,11 @@ def main():
             log(f"[bench] module: {extras['module']}")
         except Exception as e:                      # noqa: BLE001
             failures.append(f"module: {e!r}")
+        try:
+            extras["projection"] = run_projection(torch, ro, wea, ops)
+            log(f"[bench] projection: {extras['projection']}")
+        except Exception as e:                      # noqa: BLE001
+            failures.append(f"projection: {e!r}")
 
     h = per_cfg.get(head)
     result = {
