@@ -371,9 +371,12 @@ def test_clocked_entry_point_same_output_and_plausible_clocks(gpu_device):
 # ------------------------------------------------------------------------------------------
 # module-level drop-in and graph capture
 # ------------------------------------------------------------------------------------------
-def test_ring_attn_module_matches_cpu_composition(gpu_device):
+@pytest.mark.parametrize("fuse", ["none", "elementwise", "projection"])
+def test_ring_attn_module_matches_cpu_composition(gpu_device, fuse):
     """RingAttn.forward (merged QKV, GQA, value residual, head gate) against the same sequence
-    composed on the CPU from torch linears, F.rms_norm and the oracle."""
+    composed on the CPU from torch linears, F.rms_norm and the oracle - with the module's torch
+    operations around the library call, with the element-wise ones inside the kernels, and with
+    the q/k/v projection inside the store kernel as well."""
     import torch.nn.functional as F
     from types import SimpleNamespace
     torch.manual_seed(5)
@@ -383,7 +386,8 @@ def test_ring_attn_module_matches_cpu_composition(gpu_device):
                           value_residual=True, gated_attn=True)
     cos, sin = ro.rope_table_1d(16 * T, Dh)
     rope = wea.RoPE(cos, sin, 8, 8)
-    mod = wea.RingAttn(cfg, 0, rope, merged_qkv=True)
+    mod = wea.RingAttn(cfg, 0, rope, merged_qkv=True, fuse_elementwise=fuse != "none",
+                       fuse_projection=fuse == "projection")
     with torch.no_grad():
         mod.gate_proj.weight.normal_(0, 0.5)
     mod = mod.to(torch.bfloat16)
