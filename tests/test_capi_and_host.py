@@ -192,6 +192,60 @@ def test_one_call_entry_point_validates_both_halves():
     assert lib.we_rope_kv_attn_fwd(*args(extras=ctypes.byref(ex))) == -2
 
 
+def test_projection_entry_points_validate_before_launching():
+    """we_qkv_rope_kv_store / we_qkv_rope_kv_attn_fwd refuse bad operands with a status code and
+    launch nothing (no GPU is needed to see that)."""
+    lib = _capi.lib()
+    s3 = _capi.i64x3(8, 8, 8)
+    fake = ctypes.c_void_p(4096)     # never dereferenced: validation fails first
+
+    def proj(**kw):
+        pr = _capi.QkvProj()
+        pr.x, pr.w = kw.get("x", 4096), kw.get("w", 4096)
+        pr.d_model = kw.get("d_model", 256)
+        pr.x_strides = (ctypes.c_int64 * 2)(64 * 256, kw.get("xs_t", 256))
+        pr.w_row_stride = kw.get("ws", 256)
+        return pr
+
+    def store(pr, **kw):
+        return lib.we_qkv_rope_kv_store(ctypes.byref(pr) if pr is not None else None, kw.get("q_out", fake), kw.get("cos", fake),
+                                        fake, 10, fake, fake, fake, 64, 8, 8, fake, fake,
+                                        1, kw.get("H", 2), kw.get("Hkv", 2), 64, kw.get("Dh", 64), kw.get("L", 64), 1, 0,
+                                        kw.get("dtype", 0), kw.get("extras"), None)
+
+    assert store(None) == -1
+    assert store(proj(x=None)) == -1
+    assert store(proj(), q_out=None) == -1
+    assert store(proj(), cos=None) == -1               # the projection always rotates
+    assert store(proj(), L=100) == -2
+    assert store(proj(), dtype=2) == -3                # bf16 / f16 only
+    assert store(proj(), Dh=32) == -3
+    assert store(proj(d_model=192, xs_t=192, ws=192)) == -3    # contraction length not a multiple of 128
+    assert store(proj(), H=1, Hkv=1) == -3             # (H + 2 Hkv) Dh = 192 is not a whole number of feature tiles
+    assert store(proj(ws=128)) == -2                   # weight rows shorter than the contraction
+    assert store(proj(xs_t=260)) == -4                 # token stride not a multiple of 8 elements
+    ex = _capi.AttnExtras()
+    ex.v1 = 4096
+    assert store(proj(), extras=ctypes.byref(ex)) == -1        # residual without its weight
+    pr = proj()
+    rc = lib.we_qkv_rope_kv_attn_fwd(ctypes.byref(pr), fake, fake, fake, 10, fake, fake, fake, 64, 8, 8, fake, fake,
+                                     None, s3, None, 0, 1, 2, 2, 64, 64, 64, 1, 0, 0.1, 1, 0, 0, None, None)
+    assert rc == -1                                    # attention half: no output
+    rc = lib.we_qkv_rope_kv_attn_fwd(ctypes.byref(pr), fake, fake, fake, 10, fake, fake, fake, 64, 8, 8, fake, fake,
+                                     fake, s3, None, 0, 1, 2, 2, 64, 64, 64, 1, 0, 0.1, 2, 0, 0, None, None)
+    assert rc == -5                                    # splits without workspace
+    # the opaque op has a fake kernel with the module's output layouts
+    x = torch.empty(1, 64, 256, dtype=torch.bfloat16, device="meta")
+    w = torch.empty(8 * 64, 256, dtype=torch.bfloat16, device="meta")
+    kv = torch.empty(2, 1, 2, 192, 64, dtype=torch.bfloat16, device="meta")
+    written = torch.empty(192, dtype=torch.bool, device="meta")
+    t = torch.empty(1, 64, dtype=torch.long, device="meta")
+    tab = torch.empty(64, 32, device="meta")
+    y, v = torch.ops.world_engine_amd.qkv_rope_kv_attn(x, w, 4, 2, t, t, t, tab, tab, 8, 8, kv, written, 128, 1, False, 0.125)
+    assert y.shape == (1, 4, 64, 64) and y.transpose(1, 2).is_contiguous()
+    assert v.shape == (1, 2, 64, 64) and v.transpose(1, 2).is_contiguous()
+
+
 def test_attention_kernels_keep_their_state_in_registers():
     """Compile-time guard: the MFMA kernels hold accumulators, fragments and softmax state in
     VGPRs.  A source change that makes the compiler place those arrays in scratch memory still
@@ -209,6 +263,14 @@ def test_attention_kernels_keep_their_state_in_registers():
     sizes = [int(m) for m in re.findall(r"ScratchSize \[bytes/lane\]: (\d+)", r.stderr)]
     assert len(sizes) == 16, sizes          # bf16/f16 x Dh 64/128 x 128/256 queries x ragged or not
     assert max(sizes) <= 160, sizes
+    # the projection kernel: accumulators in registers, two wavefronts per SIMD
+    src = os.path.join(wbuild.CSRC, "qkv_proj_store.hip")
+    r = subprocess.run([hipcc, *[f for f in wbuild.HIPCC_FLAGS if f not in ("-shared", "-fPIC")], "-c", src, "-o", os.devnull,
+                        "--cuda-device-only", "-Rpass-analysis=kernel-resource-usage"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    sizes = [int(m) for m in re.findall(r"ScratchSize \[bytes/lane\]: (\d+)", r.stderr)]
+    vgprs = [int(m) for m in re.findall(r" VGPRs: (\d+)", r.stderr)]
+    assert len(sizes) == 2 and max(sizes) == 0 and max(vgprs) <= 256, (sizes, vgprs)
 
 
 def test_three_axis_rope_table_structure():
