@@ -190,17 +190,7 @@ def run_gpu(cfg_id, c, args, torch, ro, wea, ops):
                                  out=out, workspace=ws)
 
     if args.calibrate_copy:
-        # elementwise copy through a kernel (a same-dtype copy_() could take the DMA engines and
-        # would then be invisible to the shader counters); int32 + 0 keeps the bytes unchanged
-        n_el = args.calibrate_copy * (1 << 20) // 4
-        src = torch.arange(n_el, dtype=torch.int32, device=dev)
-        dst = torch.empty_like(src)
-        for _ in range(20):
-            torch.add(src, 0, out=dst)
-        torch.cuda.synchronize()
-        assert torch.equal(src[-4096:], dst[-4096:])
-        log(f"[bench] calibration: 20 copy kernels of {args.calibrate_copy} MiB read + {args.calibrate_copy} MiB written")
-        del src, dst
+        calibration_copies(torch, dev, args.calibrate_copy)
 
     # ---- fill the ring (untimed, not counted), then W warm-up steps ----
     for s in range(plan["first"]):
@@ -430,6 +420,21 @@ def run_module(args, torch, ro, wea):
     return res
 
 
+def calibration_copies(torch, dev, mib):
+    """20 plain copy kernels of known traffic, for scaling FETCH_SIZE / WRITE_SIZE in a counter run:
+    an elementwise copy through a kernel (a same-dtype copy_() could take the DMA engines and would
+    then be invisible to the shader counters); int32 + 0 keeps the bytes unchanged."""
+    n_el = mib * (1 << 20) // 4
+    src = torch.arange(n_el, dtype=torch.int32, device=dev)
+    dst = torch.empty_like(src)
+    for _ in range(20):
+        torch.add(src, 0, out=dst)
+    torch.cuda.synchronize()
+    assert torch.equal(src[-4096:], dst[-4096:])
+    log(f"[bench] calibration: 20 copy kernels of {mib} MiB read + {mib} MiB written")
+    del src, dst
+
+
 def run_projection(torch, ro, wea, ops):
     """The producer side of the path at cfg1's module shapes: the merged q/k/v projection + RoPE + cache
     write as the library's one kernel (we_qkv_rope_kv_store) against torch's linear layer followed by the
@@ -532,6 +537,9 @@ def main():
     ap.add_argument("--module-only", action="store_true",
                     help="only the module-level timing (RingAttn.forward at cfg1 shapes, torch and fused element-wise "
                          "neighbours): what a kernel trace of the module is taken from")
+    ap.add_argument("--projection-only", action="store_true",
+                    help="only the projection + store measurement (with --calibrate-copy: preceded by the copy kernels "
+                         "of known traffic, for a counter run)")
     ap.add_argument("--no-peaks", action="store_true", help="skip the measured GEMM / copy rates of this box")
     ap.add_argument("--two-calls", action="store_true",
                     help="we_rope_kv_store + we_attn_ring_fwd instead of the one-call we_rope_kv_attn_fwd")
@@ -556,6 +564,11 @@ def main():
     from world_engine_amd import ops
 
     torch.cuda.set_device(0)
+    if args.projection_only:
+        if args.calibrate_copy:
+            calibration_copies(torch, torch.device("cuda:0"), args.calibrate_copy)
+        print(json.dumps({"projection": run_projection(torch, ro, wea, ops)}), flush=True)
+        return
     if args.module_only:
         print(json.dumps({"module": run_module(args, torch, ro, wea),
                           "projection": run_projection(torch, ro, wea, ops)}), flush=True)
