@@ -43,8 +43,9 @@ def test_one_call_schedule_small_frames(gpu_device, dtype, Dh):
             assert_attn_close(out, ref, f"t={t} sub={sub}")
 
 
-def test_one_call_cfg1_shape(gpu_device):
-    p = Pair(gpu_device, torch.bfloat16, B=1, H=16, Hkv=16, T=256, Dh=128, n_slots=16, cfg_id=1)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_one_call_cfg1_shape(gpu_device, dtype):
+    p = Pair(gpu_device, dtype, B=1, H=16, Hkv=16, T=256, Dh=128, n_slots=16, cfg_id=1)
     for t in list(range(0, 20)) + [31, 32, 33]:
         out, ref = _one_call_step(p, t, 0, False)
         assert_attn_close(out, ref, f"t={t}")
