@@ -274,9 +274,10 @@ int we_rope_kv_attn_fwd(const void* q, const void* k, const void* v,
  *                [B, Hkv, T, Dh] with element strides v_out_strides = {batch, head, token} - what
  *                the first layer hands on as `v1` (src/model/attn.py:107).  NULL = not wanted.
  * The projection accumulates in fp32 and rounds once to the element type, like the GEMM's output
- * tensor; sums are taken in a fixed order (results are reproducible, and exact whenever the fp32
- * sums are exact) that differs from a BLAS library's, i.e. rows may differ from
- * torch.nn.functional.linear's in the last bit of the element type.  bf16 / f16 only;
+ * tensor; sums are taken in an order fixed by the shapes and the token's 64-token tile (results
+ * are reproducible, and exact whenever the fp32 sums are exact) that differs from a BLAS
+ * library's, i.e. rows may differ from torch.nn.functional.linear's in the last bit of the
+ * element type.  bf16 / f16 only;
  * (H + 2 Hkv) * Dh must be a multiple of 128 and Dh 64 or 128.
  */
 typedef struct we_qkv_proj {

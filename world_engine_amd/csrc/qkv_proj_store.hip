@@ -114,8 +114,15 @@ qkv_rope_store_kernel(ProjParams p) {
   constexpr int NDMA = 6;  // DMA instructions per wavefront and slot
 
   const int nc = p.K / PK;
-  dma_slot(0, 0);
-  if (nc > 1) dma_slot(1, 1);
+  // Contraction chunks are taken four at a time, and within a group of four token tile i starts at
+  // chunk i: the tiles that share a weight slab then ask for different lines at any one time, each
+  // line comes from HBM at one tile's request and is an L2 hit for the other three a slot or two
+  // later.  (A CU streams from HBM at less than half the rate it reads L2 at, so four tiles asking
+  // for the same lines together move the slab at a quarter of what they could.)
+  const int rot = mi & 3, nc4 = nc & ~3;
+  auto chunk = [&](int c) __attribute__((always_inline)) { return c < nc4 ? (c & ~3) | ((c + rot) & 3) : c; };
+  dma_slot(chunk(0), 0);
+  if (nc > 1) dma_slot(chunk(1), 1);
 
   // ---- what the item needs besides the projection: requested now, used after the loop ----
   ItemSide<Tag> side;
@@ -146,7 +153,7 @@ qkv_rope_store_kernel(ProjParams p) {
     // every wavefront's part has landed, and everybody is done with the slot refilled next
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    if (c + 2 < nc) dma_slot(c + 2, fill);
+    if (c + 2 < nc) dma_slot(chunk(c + 2), fill);
     fill = fill + 1 == NSLOT ? 0 : fill + 1;
 #pragma unroll
     for (int h2 = 0; h2 < 2; ++h2) {
