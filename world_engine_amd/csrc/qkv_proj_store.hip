@@ -114,13 +114,15 @@ qkv_rope_store_kernel(ProjParams p) {
   constexpr int NDMA = 6;  // DMA instructions per wavefront and slot
 
   const int nc = p.K / PK;
-  // Contraction chunks are taken four at a time, and within a group of four token tile i starts at
-  // chunk i: the tiles that share a weight slab then ask for different lines at any one time, each
-  // line comes from HBM at one tile's request and is an L2 hit for the other three a slot or two
-  // later.  (A CU streams from HBM at less than half the rate it reads L2 at, so four tiles asking
-  // for the same lines together move the slab at a quarter of what they could.)
-  const int rot = mi & 3, nc4 = nc & ~3;
-  auto chunk = [&](int c) __attribute__((always_inline)) { return c < nc4 ? (c & ~3) | ((c + rot) & 3) : c; };
+  // Contraction chunks are taken in groups of G, and within a group token tile i starts at chunk
+  // i mod G: the tiles that share a weight slab then ask for different lines at any one time, each
+  // line comes from HBM at one tile's request and is an L2 hit for the others a slot or two later.
+  // (A CU streams from HBM at less than half the rate it reads L2 at, so tiles asking for the same
+  // lines together move the slab at a fraction of what they could.  Groups longer than 8 slots
+  // keep more of the slab alive in L2 than pays.)
+  const int G = mt_all >= 8 ? 8 : (mt_all >= 4 ? 4 : (mt_all >= 2 ? 2 : 1));
+  const int rot = mi & (G - 1), ncg = nc & ~(G - 1);
+  auto chunk = [&](int c) __attribute__((always_inline)) { return c < ncg ? (c & ~(G - 1)) | ((c + rot) & (G - 1)) : c; };
   dma_slot(chunk(0), 0);
   if (nc > 1) dma_slot(chunk(1), 1);
 
