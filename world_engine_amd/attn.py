@@ -160,6 +160,9 @@ class RingAttn(nn.Module):
         self.enable_gqa = self.n_heads != self.n_kv_heads
         self.q_out = self.n_heads * self.d_head
         self.kv_out = self.n_kv_heads * self.d_head
+        if fuse_projection and (config.d_model % 128 or (self.q_out + 2 * self.kv_out) % 128 or self.d_head not in (64, 128)):
+            raise AssertionError("fuse_projection needs d_model and (n_heads + 2 n_kv_heads) * d_head to be multiples "
+                                 "of 128 and a head dim of 64 or 128")
 
         self.value_residual = getattr(config, "value_residual", False)
         if self.value_residual:
