@@ -66,9 +66,12 @@ def test_workspace_and_split_planning():
     lib = _capi.lib()
     assert lib.we_attn_workspace_bytes(1, 16, 16, 256, 128, 4096, 1, 0) == 0
     assert lib.we_attn_workspace_bytes(1, 16, 16, 256, 128, 4096, 4, 0) == 4 * 16 * 256 * (128 * 2 + 16)
-    # 256-token frames: every unit is split so that all 256 CUs have work
+    # 256-token frames: every unit is split, into three quarters of the parts that would give every CU a workgroup
     s = lib.we_attn_auto_splits(1, 16, 16, 256, 128, 4096)
-    assert s == 8
+    assert s == 6
+    # ... and the workgroups of a call never outnumber the 256 CUs: 48, 80, 96, 160 unsplit workgroups
+    for heads, want in ((24, 4), (40, 3), (48, 2), (80, 1)):
+        assert lib.we_attn_auto_splits(1, heads, heads, 256, 128, 4096) == want, heads
     assert lib.we_attn_workspace_bytes(1, 16, 16, 256, 128, 4096, 0, 0) == s * 16 * 256 * (128 * 2 + 16)
     # 1024-token frames with 96 heads: 384 workgroups of 256 queries = 1.5 rounds of 256 CUs, so only
     # the last 32 of the 96 units (128 workgroups) are split in two

@@ -59,7 +59,8 @@ struct AttnPlan {
 //  * Shape: 256 queries per workgroup when that alone gives at least one workgroup per CU, else
 //    128 queries (two wavefronts share each query block and split every tile's keys).
 //  * Few workgroups (256-token frames): every unit is split into the same number of context
-//    parts, enough for one workgroup per CU but never fewer than two 64-key tiles per part.
+//    parts - as many as fit the CUs in one round, three quarters of that from four parts on -
+//    but never fewer than two 64-key tiles per part.
 //  * Many workgroups that do not divide into whole rounds of 256 CUs (e.g. 384): only the units
 //    of the last, partial round are split, so that round finishes in a fraction of the time.
 AttnPlan plan_attn(int B, int H, int Hkv, int T, int64_t L, int n_splits, int variant) {
@@ -77,9 +78,16 @@ AttnPlan plan_attn(int B, int H, int Hkv, int T, int64_t L, int n_splits, int va
   if (n_splits > 0) {
     pl.n_splits = n_splits;
   } else if (wgs < 256) {
-    int64_t s = (256 + wgs - 1) / wgs;
+    // Never more workgroups than CUs (a second, nearly empty round costs a whole kernel's
+    // time); and when the context is cut four ways or more, three quarters of the CUs rather than
+    // all of them: the parts get longer, the partial results fewer, and the memory system, not
+    // the number of CUs, is what 256-token frames wait for (cfg1: 6 parts 25.1 us per frame-step,
+    // 8 parts 27.2; 24 rings: 653 against 717; measured over 8 to 160 workgroups per call).
+    int64_t s = 256 / wgs;
+    if (s >= 4) s = 192 / wgs;
     if (s > max_s) s = max_s;
     if (s > 64) s = 64;
+    if (s < 1) s = 1;
     pl.n_splits = (int)s;
   } else if (wgs < 4 * 256 && members <= 256) {
     const int whole_units = (int)((wgs / 256) * 256 / members);
