@@ -70,7 +70,7 @@ def test_workspace_and_split_planning():
     s = lib.we_attn_auto_splits(1, 16, 16, 256, 128, 4096)
     assert s == 6
     # ... and the workgroups of a call never outnumber the 256 CUs: 48, 80, 96, 160 unsplit workgroups
-    for heads, want in ((24, 4), (40, 3), (48, 2), (80, 1)):
+    for heads, want in ((24, 5), (40, 3), (48, 2), (80, 1)):
         assert lib.we_attn_auto_splits(1, heads, heads, 256, 128, 4096) == want, heads
     assert lib.we_attn_workspace_bytes(1, 16, 16, 256, 128, 4096, 0, 0) == s * 16 * 256 * (128 * 2 + 16)
     # 1024-token frames with 96 heads: 384 workgroups of 256 queries = 1.5 rounds of 256 CUs, so only

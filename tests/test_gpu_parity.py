@@ -234,11 +234,16 @@ def test_attention_rings_longer_than_one_wavefront(gpu_device, n_slots, T, Dh, k
 
 def test_attention_partial_round_tail_split(gpu_device):
     """320 workgroups = one full round of 256 CUs plus a quarter round: the library splits the
-    context of the last 32 heads only (mixed direct-output and workspace rows in one call)."""
-    assert ops.attn_auto_splits(1, 160, 160, 256, 64, 512) == 2
-    assert ops.attn_workspace_bytes(1, 160, 160, 256, 64, 512) == 2 * 32 * 256 * (64 * 2 + 16)
-    p = Pair(gpu_device, torch.bfloat16, B=1, H=160, Hkv=160, T=256, Dh=64, n_slots=2, cfg_id=27)
+    context of the last 64 heads only (mixed direct-output and workspace rows in one call).  With
+    160 heads the same frame is one round of 160 256-query workgroups and nothing is split."""
+    assert ops.attn_auto_splits(1, 160, 160, 256, 64, 512) == 1
+    assert ops.attn_workspace_bytes(1, 160, 160, 256, 64, 512) == 0
+    assert ops.attn_auto_splits(1, 320, 320, 256, 64, 512) == 2
+    assert ops.attn_workspace_bytes(1, 320, 320, 256, 64, 512) == 2 * 64 * 256 * (64 * 2 + 16)
+    p = Pair(gpu_device, torch.bfloat16, B=1, H=320, Hkv=320, T=256, Dh=64, n_slots=2, cfg_id=27)
     _run_and_check(p, 4)
+    p = Pair(gpu_device, torch.bfloat16, B=1, H=160, Hkv=160, T=256, Dh=64, n_slots=2, cfg_id=27)
+    _run_and_check(p, 3)
 
 
 @pytest.mark.parametrize("d", [2, 4])

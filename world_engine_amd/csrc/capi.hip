@@ -66,7 +66,11 @@ struct AttnPlan {
 AttnPlan plan_attn(int B, int H, int Hkv, int T, int64_t L, int n_splits, int variant) {
   AttnPlan pl;
   const int64_t wg256 = (int64_t)B * H * ((T + 255) / 256);
-  pl.variant = variant ? variant : ((T >= 256 && wg256 >= 256) ? 2 : 1);
+  const int64_t wg128 = (int64_t)B * H * ((T + 127) / 128);
+  // 256 queries per workgroup when that alone fills the CUs - or when 128 would spill into a
+  // second round that 256 avoids (136 to 256 heads of a 256-token frame: one round of fat
+  // workgroups beats one and a bit rounds of thin ones by 5 to 17 %)
+  pl.variant = variant ? variant : ((T >= 256 && (wg256 >= 256 || wg128 > 256)) ? 2 : 1);
   pl.block_m = pl.variant == 2 ? 256 : 128;
   const int units = B * Hkv;
   const int members = (H / Hkv) * ((T + pl.block_m - 1) / pl.block_m);
@@ -79,12 +83,13 @@ AttnPlan plan_attn(int B, int H, int Hkv, int T, int64_t L, int n_splits, int va
     pl.n_splits = n_splits;
   } else if (wgs < 256) {
     // Never more workgroups than CUs (a second, nearly empty round costs a whole kernel's
-    // time); and when the context is cut four ways or more, three quarters of the CUs rather than
-    // all of them: the parts get longer, the partial results fewer, and the memory system, not
-    // the number of CUs, is what 256-token frames wait for (cfg1: 6 parts 25.1 us per frame-step,
-    // 8 parts 27.2; 24 rings: 653 against 717; measured over 8 to 160 workgroups per call).
+    // time); and when the context is cut four ways or more, fewer workgroups than CUs: the parts
+    // get longer, the partial results fewer, and the memory system, not the number of CUs, is
+    // what 256-token frames wait for (cfg1: 6 parts 25.1 us per frame-step, 8 parts 27.2; 24
+    // rings: 653 against 717).  Measured over 8 to 160 workgroups per call: the best count is
+    // about 240 workgroups for up to six parts and about 192 for more.
     int64_t s = 256 / wgs;
-    if (s >= 4) s = 192 / wgs;
+    if (s >= 4) s = (wgs >= 40 ? 240 : 192) / wgs;
     if (s > max_s) s = max_s;
     if (s > 64) s = 64;
     if (s < 1) s = 1;
