@@ -517,6 +517,24 @@ def run_peaks(torch):
     t_cp = timed(lambda: torch.add(src, 0, out=dst), 20)
     peaks = {"bf16_gemm_8192_tflops": round(2 * 8192 ** 3 / t_mm / 1e12, 1),
              "copy_1gib_read_plus_write_gbps": round(2 * src.numel() * 4 / t_cp / 1e9, 1)}
+    # The same copy kernel at the size of one attention call's traffic (cfg1 moves 35.7 MB, cfg4
+    # 69.2 MB), launched back to back from a HIP graph as the attention calls are: what a kernel
+    # that does nothing but move that many bytes reaches here, launch and ramp included.
+    for mib in (32, 64):
+        n = mib * (1 << 20) // 8   # int32 elements read; as many written
+        s_, d_ = src[:n], dst[:n]
+        for _ in range(3):
+            torch.add(s_, 0, out=d_)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(50):
+                torch.add(s_, 0, out=d_)
+        g.replay()
+        torch.cuda.synchronize()
+        t = timed(g.replay, 5) / 50
+        peaks[f"copy_{mib}mib_moved_us"] = round(t * 1e6, 2)
+        peaks[f"copy_{mib}mib_moved_gbps"] = round(mib * (1 << 20) / t / 1e9, 1)
     del a, b2, src, dst
     torch.cuda.empty_cache()
     return peaks
