@@ -155,6 +155,25 @@ def test_attention_module_parameters_and_casting():
     assert wea.install_ring_attention(m, rope, (Legacy,)) == 0
 
 
+def test_fused_projection_is_chosen_by_shape():
+    """fuse_projection runs the library's projection kernel where its workgroups (64 tokens x
+    128 features each) fit the CUs in one round, and the linear layer + store call beyond."""
+    rope = wea.RoPE.one_dimensional(128, 128, 16, 16)
+    cfg = SimpleNamespace(n_heads=16, n_kv_heads=16, d_model=2048)
+    m = wea.RingAttn(cfg, 0, rope, merged_qkv=True, fuse_elementwise=True, fuse_projection=True)
+    assert m.projection_workgroups(1, 256) == 4 * 48 and m.uses_fused_projection(1, 256)
+    assert m.projection_workgroups(1, 264) == 5 * 48 and m.uses_fused_projection(1, 264)
+    assert m.projection_workgroups(1, 1024) == 16 * 48 and not m.uses_fused_projection(1, 1024)
+    assert not m.uses_fused_projection(4, 256)
+    assert m.uses_fused_projection(1, 8)
+    plain = wea.RingAttn(cfg, 0, rope, merged_qkv=True, fuse_elementwise=True)
+    assert not plain.uses_fused_projection(1, 256)
+    wide = wea.RingAttn(SimpleNamespace(n_heads=24, n_kv_heads=24, d_model=3072), 0, rope, merged_qkv=True,
+                        fuse_elementwise=True, fuse_projection=True)
+    assert wide.projection_workgroups(1, 256) == 288 and not wide.uses_fused_projection(1, 256)
+    assert wide.uses_fused_projection(1, 192)
+
+
 def test_custom_ops_registered_with_fake_kernels():
     q = torch.empty(1, 4, 64, 64, dtype=torch.bfloat16, device="meta")
     kv = torch.empty(2, 1, 4, 192, 64, dtype=torch.bfloat16, device="meta")

@@ -184,6 +184,45 @@ def test_module_with_fused_projection(gpu_device, compiled):
             assert torch.equal(caches[1].layers[li].written, caches[0].layers[li].written)
 
 
+def test_module_takes_the_linear_layer_beyond_one_round_of_workgroups(gpu_device):
+    """1024-token frames of 16 heads need 768 projection workgroups: RingAttn(fuse_projection=True)
+    takes the linear layer + the fuse_elementwise call there, so it matches the module built
+    without fuse_projection bit for bit; a 256-token frame of the same module (192 workgroups)
+    takes the projection kernel and agrees to rounding."""
+    import types
+    import world_engine_amd as wea
+    torch.manual_seed(5)
+    dev = gpu_device
+    cos, sin = ro.rope_table_1d(8 * 1024, 128)
+    for T, side in ((1024, 32), (256, 16)):
+        cfg = types.SimpleNamespace(d_model=2048, n_heads=16, n_kv_heads=16, value_residual=False, gated_attn=False,
+                                    tokens_per_frame=T, local_window=2, global_window=2, global_attn_period=1,
+                                    global_pinned_dilation=1, n_layers=1)
+        rope = wea.RoPE(cos, sin, side, side).to(dev)
+        plain = wea.RingAttn(cfg, 0, rope, merged_qkv=True, fuse_elementwise=True).to(dev, torch.bfloat16)
+        fused = wea.RingAttn(cfg, 0, rope, merged_qkv=True, fuse_elementwise=True, fuse_projection=True).to(dev, torch.bfloat16)
+        fused.load_state_dict(plain.state_dict())
+        assert fused.uses_fused_projection(1, T) == (T == 256)
+        caches = [wea.StaticKVCache(cfg, 1, torch.bfloat16).to(dev) for _ in range(2)]
+        for c in caches:
+            c.set_frozen(False)
+        for t in range(3):
+            print(f"shape rule T={T} t={t}", flush=True)
+            x = torch.randn(1, T, 2048, device=dev, dtype=torch.bfloat16)
+            pos = to_dev(ro.synth_pos_ids(t, 1, T, side), dev)
+            with torch.no_grad():
+                ya, _ = plain(x, pos, None, caches[0])
+                yb, _ = fused(x, pos, None, caches[1])
+            if T == 1024:
+                assert torch.equal(ya, yb), t
+                assert torch.equal(caches[0].layers[0].kv, caches[1].layers[0].kv), t
+            else:
+                assert_ulp_close(caches[1].layers[0].kv, caches[0].layers[0].kv, f"cache t={t}")
+                d = (ya.float() - yb.float()).abs().max().item()
+                assert d <= 2e-2 * max(1.0, ya.float().abs().max().item()), (t, d)
+            assert torch.equal(caches[0].layers[0].written, caches[1].layers[0].written)
+
+
 def _proj_case(seed):
     import random
     r = random.Random(1000 + seed)

@@ -141,7 +141,18 @@ class RingAttn(nn.Module):
     q/k/v projection in the library, in one kernel with the cache write: x goes in, the rotated q
     and the cache rows come out, the ``[B, T, (H + 2 Hkv) Dh]`` projection output never exists.
     Its rows are fp32 sums rounded once like the BLAS routine's, in another order of additions.
+    That kernel is built for the frames this path is slow on - a few hundred tokens, where the
+    projection streams its weights once and is bound by memory latency: 64 tokens x 128 features
+    per workgroup, one workgroup per CU.  Where the shape needs more workgroups than the 256 CUs
+    (``fused_projection_max_workgroups``) the projection is a matrix-core-bound GEMM, the BLAS
+    routine is the faster one (measured at 16 heads of 128, d_model 2048, per call: 256 tokens
+    16.5 us against 23.4 us for linear layer + store kernel; 1024 tokens 45 against 36; 4096
+    tokens of 24 heads, d_model 3072: 356 against 214), and ``forward`` takes the linear layer
+    followed by the ``fuse_elementwise`` call instead.
     """
+
+    # one round of workgroups on the 256 CUs of an MI355X
+    fused_projection_max_workgroups = 256
 
     def __init__(self, config, layer_idx: int, rope: RoPE, merged_qkv: bool = False,
                  fuse_elementwise: bool = False, fuse_projection: bool = False):
@@ -215,9 +226,16 @@ class RingAttn(nn.Module):
             v1 = v
         return self.out_proj(y.transpose(1, 2).reshape(B, T, -1)), v1
 
+    def projection_workgroups(self, B: int, T: int) -> int:
+        """Workgroups the fused projection kernel launches for x ``[B, T, d_model]``."""
+        return B * ((T + 63) // 64) * ((self.q_out + 2 * self.kv_out) // 128)
+
+    def uses_fused_projection(self, B: int, T: int) -> bool:
+        return self.fuse_projection and self.projection_workgroups(B, T) <= self.fused_projection_max_workgroups
+
     def forward(self, x: Tensor, pos_ids: Mapping[str, Tensor], v1: Optional[Tensor], kv_cache):
         B, T = x.shape[:2]
-        if (self.fuse_projection and hasattr(kv_cache, "qkv_rope_upsert_attend")
+        if (self.uses_fused_projection(B, T) and hasattr(kv_cache, "qkv_rope_upsert_attend")
                 and x.dtype in (torch.bfloat16, torch.float16) and x.stride(-1) == 1):
             return self._forward_fused_projection(x, pos_ids, v1, kv_cache)
         if self.merged_qkv:
