@@ -535,6 +535,24 @@ def run_peaks(torch):
         t = timed(g.replay, 5) / 50
         peaks[f"copy_{mib}mib_moved_us"] = round(t * 1e6, 2)
         peaks[f"copy_{mib}mib_moved_gbps"] = round(mib * (1 << 20) / t / 1e9, 1)
+    # The attention kernel's own K/V tile stream at 256-token frames without the arithmetic
+    # (we_stream_probe): 192 workgroups, two per stream, 23 (cfg1) or 45 (cfg4) 16-KB tiles each.
+    from world_engine_amd import ops
+    for name, tiles in (("cfg1", 23), ("cfg4", 45)):
+        nbytes = 96 * tiles * 16384
+        ring = src.view(torch.uint8)[:nbytes]
+        for _ in range(3):
+            ops.stream_probe(ring, 192, tiles, 2)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(50):
+                ops.stream_probe(ring, 192, tiles, 2)
+        g.replay()
+        torch.cuda.synchronize()
+        t = timed(g.replay, 5) / 50
+        peaks[f"tile_stream_{name}_us"] = round(t * 1e6, 2)
+        peaks[f"tile_stream_{name}_gbps"] = round(nbytes / t / 1e9, 1)
     del a, b2, src, dst
     torch.cuda.empty_cache()
     return peaks

@@ -178,6 +178,19 @@ int we_attn_ring_fwd_clocked(const void* q, const int64_t q_strides[3],
                              int32_t dtype, uint64_t* clocks, size_t clocks_len, void* stream);
 
 /*
+ * Measurement aid without a counterpart in the reference: the attention kernel's way of fetching
+ * K and V tiles at 256-token frames with the arithmetic taken away.  `workgroups` workgroups (one
+ * per CU, a multiple of 8: workgroup id % 8 is the XCD) each stream `tiles` 16-KB tiles of one
+ * contiguous region of `buf` into LDS by DMA, three tiles in flight, one barrier per tile;
+ * `share` consecutive workgroups of an XCD walk the same region (the query tiles and grouped heads
+ * of one K/V stream).  Region r starts at byte r * tiles * 16384; buf_bytes must cover the
+ * workgroups / share regions (WE_ERR_WORKSPACE otherwise).  Nothing is written.  The duration of a
+ * launch is the floor for a kernel of this shape, whatever it computes.
+ */
+int we_stream_probe(const void* buf, size_t buf_bytes, int32_t workgroups, int32_t tiles, int32_t share,
+                    void* stream);
+
+/*
  * we_attn_ring_fwd for callers that cannot allocate device memory, not even a workspace: code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
  * counterpart in the reference (whose attention call allocates through torch as it pleases).

@@ -344,6 +344,47 @@ def test_output_layout_and_out_argument(gpu_device):
     assert c.data_ptr() == out.data_ptr() and torch.equal(out, b)
 
 
+@pytest.mark.parametrize("T,Dh", [(256, 128), (72, 64)])
+def test_query_rows_far_apart_take_the_register_path(gpu_device, T, Dh):
+    """128-query workgroups fetch their Q tile by DMA with 32-bit row offsets; a q whose rows lie
+    more than 2 GiB / T apart (here: a view into a 2.1 GB buffer) has its fragments loaded lane by
+    lane instead.  Same values, same arithmetic: the outputs must be bit-identical."""
+    _say(f"far-apart query rows T={T} Dh={Dh}")
+    H = 2
+    p = Pair(gpu_device, torch.bfloat16, B=1, H=H, Hkv=1, T=T, Dh=Dh, n_slots=3, cfg_id=27)
+    row = (1 << 31) // (2 * T) + 64                  # elements between two tokens' rows
+    far = torch.empty(T, row, dtype=torch.bfloat16, device=gpu_device)
+    for t in range(4):
+        p.set_frozen(t == 2)
+        q, k, v, pos = p.inputs(t)
+        (q_o, k_all, v_all, mask), (q_h, ring) = p.store(q, k, v, pos)
+        far[:, : H * Dh] = q_h.transpose(1, 2).reshape(T, H * Dh)
+        q_far = far[:, : H * Dh].view(1, T, H, Dh).transpose(1, 2)
+        assert q_far.stride(2) * T * 2 >= 1 << 31
+        for kw in ({"q_tile": 128}, {"q_tile": 128, "n_splits": 2}):
+            a = p.attend(q_h, ring, **kw)
+            b = p.attend(q_far, ring, **kw)
+            assert torch.equal(a, b), (t, kw)
+        assert_attn_close(a, ro.attention_fp32(q_o, k_all, v_all, mask), f"t={t}")
+
+
+def test_stream_probe_runs_and_validates(gpu_device):
+    """The tile-stream measurement aid: launches on a buffer that covers its regions, refuses one
+    that does not, and writes nothing."""
+    _say("stream probe")
+    buf = torch.full((96 * 23 * 16384,), 7, dtype=torch.uint8, device=gpu_device)
+    ops.stream_probe(buf, 192, 23, 2)
+    ops.stream_probe(buf, 8, 1, 1)
+    torch.cuda.synchronize()
+    assert bool((buf == 7).all())
+    with pytest.raises(RuntimeError, match="we_stream_probe"):
+        ops.stream_probe(buf, 192, 23, 1)            # 192 regions do not fit
+    with pytest.raises(RuntimeError, match="we_stream_probe"):
+        ops.stream_probe(buf, 100, 23, 2)            # not a multiple of 8 workgroups
+    with pytest.raises(RuntimeError, match="we_stream_probe"):
+        ops.stream_probe(buf, 192, 0, 2)
+
+
 def test_clocked_entry_point_same_output_and_plausible_clocks(gpu_device):
     """``we_attn_ring_fwd_clocked`` is ``we_attn_ring_fwd`` plus two counters per workgroup: the
     output has the same bits, every workgroup reports a duration, and cycles per 100 MHz tick is a

@@ -74,6 +74,7 @@ SIGNATURES = {
         c_int32, c_float, c_int32, c_int32, c_int32,            # dilation scale n_splits q_tile dtype
         c_void_p, c_size_t, c_void_p,              # clocks, clocks_len, stream
     ]),
+    "we_stream_probe": (c_int32, [c_void_p, c_size_t, c_int32, c_int32, c_int32, c_void_p]),
     "we_attn_ring_fwd_static": (c_int32, [
         c_void_p, _I64x3,                          # q, q_strides
         c_void_p, c_void_p, c_void_p,              # kv, written, t_pos

@@ -21,6 +21,7 @@ UNITS = [("rope_kv_store.hip", [], "rope_kv_store.o"),
          ("attn_ring.hip", ["-DWE_RING_PART=3"], "attn_ring_f16_64.o"),
          ("attn_ring_f32.hip", [], "attn_ring_f32.o"),
          ("attn_combine.hip", [], "attn_combine.o"),
+         ("stream_probe.hip", [], "stream_probe.o"),
          ("capi.hip", [], "capi.o")]
 SOURCES = sorted({u[0] for u in UNITS})
 OUT = os.path.join(HERE, "libwe_attn.so")

@@ -148,9 +148,17 @@ attn_ring_kernel(AttnParams p) {
   const int h = hkv * p.group + hq_in;
 
   // ---- raw Q fragments ----
+  // A lane's fragment loads touch 32 rows x 32 bytes each: 512 small requests per wavefront, which
+  // the 256-query shape (long loops) does not notice and the 128-query shape does: the tile DMAs
+  // below cannot go out before Q is back.  There the workgroup's 128 x Dh tile comes by DMA - 16
+  // lanes per row, whole cache lines - into the V ring's slots 2 and 3, laid out and swizzled like
+  // two K tiles, while the slot flags are on their way; the fragments are read from there once the
+  // first K tile is in, and slot 3 is zeroed afterwards.
+  constexpr int Q_OFF = L::V_OFF + 2 * TILE_B;
+  const bool q_dma = KSPLIT == 2 && p.q_dma != 0;
   frag_t qf[KS];
   const int qrow = qtile * BM + qb * 32 + l32;
-  {
+  if (!q_dma) {
     const uint16_t* qbase = reinterpret_cast<const uint16_t*>(p.q) + b * p.qs_b + h * p.qs_h;
     const int qr = qrow < p.T ? qrow : p.T - 1;
     const uint16_t* src = qbase + (int64_t)qr * p.qs_t + hh * 8;
@@ -158,6 +166,17 @@ attn_ring_kernel(AttnParams p) {
     for (int ks = 0; ks < KS; ++ks) qf[ks] = *reinterpret_cast<const frag_t*>(src + ks * 16);
   }
   if (us_raw >= p.unit_splits) return;
+  if (KSPLIT == 2 && q_dma) {
+    const uint64_t qplane = uniform64((uint64_t)(uintptr_t)p.q + (uint64_t)(((int64_t)b * p.qs_b + (int64_t)h * p.qs_h) * 2));
+    const uint32_t q_lds = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds0 + Q_OFF + wave * 1024));
+#pragma unroll
+    for (int i = 0; i < 2 * NDMA; ++i) {
+      const int row = (wave + i * 8) * RPI + lane / CPR;   // row of the 128-query tile
+      int qr = qtile * BM + row;
+      qr = qr < p.T ? qr : p.T - 1;
+      dma16(qplane, (uint32_t)qr * (uint32_t)(p.qs_t * 2) + (uint32_t)(((lane % CPR) ^ k_swz<DH>(row)) << 4), q_lds + i * 8 * 1024);
+    }
+  }
 
   // ---- list of visible slots (the tail is pseudo-slot n_slots) ----
   // Every wavefront builds it for itself (no barrier, no serial section) in a private strip of
@@ -476,11 +495,15 @@ attn_ring_kernel(AttnParams p) {
   };
 
   if (ntile > 0) {
-    {
-      // zero V slot 3, which stands in for "tile -1", and P, so the first product adds zeros
+    // zero V slot 3, which stands in for "tile -1", and P, so the first product adds zeros
+    auto zero_v3 = [&]() __attribute__((always_inline)) {
       const u32x4_t z = {0u, 0u, 0u, 0u};
       unsigned char* vz = smem + L::V_OFF + 3 * TILE_B;
       for (int i = tid; i < TILE_B / 16; i += 512) *reinterpret_cast<u32x4_t*>(vz + i * 16) = z;
+    };
+    if (!q_dma) zero_v3();  // (with the Q tile staged there: once its fragments have been read)
+    {
+      const u32x4_t z = {0u, 0u, 0u, 0u};
       p_prev[0] = __builtin_bit_cast(frag_t, z);
       p_prev[1] = __builtin_bit_cast(frag_t, z);
     }
@@ -493,8 +516,10 @@ attn_ring_kernel(AttnParams p) {
     uint32_t off1, off2;  // offsets of the last and the last-but-one tile the K stream visited
     // Q was requested before the slot flags and loads return in order, so it is here; stating a
     // use now keeps the wait for it from landing behind the tile DMAs issued next.
+    if (!q_dma) {
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) asm volatile("" ::"v"(qf[ks]));
+      for (int ks = 0; ks < KS; ++ks) asm volatile("" ::"v"(qf[ks]));
+    }
     {
       const uint32_t o0 = next_off();
       const uint32_t o1 = next_off();
@@ -513,9 +538,16 @@ attn_ring_kernel(AttnParams p) {
       }
       dma_v(o1, 1);
     }
-    // (Q stays in registers for the whole kernel, as loaded)
     dma_wait<(KA + 1) * NDMA>();
-    __syncthreads();  // K(0) and the zeroed V slot are in LDS
+    __syncthreads();  // K(0) and the zeroed V slot (or the Q tile, requested long before K(0)) are in LDS
+    if (KSPLIT == 2 && q_dma) {
+      // row qb*32 + l32 of the tile, logical chunk 2*ks + hh: the K fragment's address arithmetic
+      const int x = k_swz<DH>(l32);
+      const uint32_t q_rd = (uint32_t)(Q_OFF + qb * KB_B + l32 * ROW_B + ((((x >> 1) << 1) | (hh ^ (x & 1))) << 4));
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) qf[ks] = *reinterpret_cast<const frag_t*>(smem + (q_rd ^ (ks << 5)));
+    }
+    // (Q stays in registers for the rest of the kernel)
     // first block: reference = its row max
     {
       s_cur = zero16;
@@ -533,6 +565,10 @@ attn_ring_kernel(AttnParams p) {
         cur_keys = nk0;
       }
       set_shift();
+    }
+    if (KSPLIT == 2 && q_dma) {
+      __syncthreads();  // every wavefront has its Q fragments: the staging area becomes V slots again
+      zero_v3();
     }
     dma_wait<2 * NDMA>();
     __syncthreads();  // everything but the last K and V tile issued so far has landed
@@ -607,6 +643,8 @@ attn_ring_kernel(AttnParams p) {
       }
     }
     dma_wait<0>();  // no DMA may still be writing LDS when the rings are reused or the CU is freed
+  } else if (q_dma) {
+    dma_wait<0>();  // (a split without visible keys: the Q tile it asked for must not land after the merge below)
   }
 
   float lo, up;

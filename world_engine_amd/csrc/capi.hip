@@ -210,6 +210,7 @@ int prepare_attn(const void* q, const int64_t* q_strides, const void* kv, const 
   p.gate = nullptr; p.gs_b = p.gs_h = p.gs_t = 0;
   p.gate_x = nullptr; p.gate_w = nullptr; p.gx_b = p.gx_t = 0;
   p.clock_out = nullptr;
+  p.q_dma = (q_strides[2] > 0 && (uint64_t)T * (uint64_t)q_strides[2] * 2u < (1ull << 31)) ? 1 : 0;
 
   if ((p.unit_splits + 7) / 8 > 65535 || p.group > 65535 || (int64_t)B * H - (int64_t)pl.units_whole * p.group > 65535)
     return WE_ERR_UNSUPPORTED;  // grid y / z limits of the two launches
@@ -411,6 +412,19 @@ int we_attn_ring_fwd_clocked(const void* q, const int64_t q_strides[3], const vo
   if (clocks_len < 2 * wgs) return WE_ERR_WORKSPACE;
   p.clock_out = clocks;
   return launch_attn(p, pl, Dh, dtype, static_cast<hipStream_t>(stream));
+}
+
+int we_stream_probe(const void* buf, size_t buf_bytes, int32_t workgroups, int32_t tiles, int32_t share, void* stream) {
+  if (!buf) return WE_ERR_NULL_POINTER;
+  if (workgroups <= 0 || workgroups % 8 != 0 || workgroups > 65536 || tiles <= 0 || tiles > 65536 || share <= 0 ||
+      (workgroups / 8) % share != 0)
+    return WE_ERR_BAD_SHAPE;
+  if (!aligned16(buf)) return WE_ERR_ALIGNMENT;
+  const uint64_t region = (uint64_t)tiles * 16384u;
+  if (region >= (1ull << 32)) return WE_ERR_UNSUPPORTED;  // 32-bit DMA offsets within a region
+  if ((uint64_t)(workgroups / share) * region > buf_bytes) return WE_ERR_WORKSPACE;
+  return we::launch_stream_probe(buf, workgroups, tiles, share, static_cast<hipStream_t>(stream)) == hipSuccess
+             ? WE_OK : WE_ERR_LAUNCH;
 }
 
 int we_attn_ring_fwd_static(const void* q, const int64_t q_strides[3], const void* kv, const uint8_t* written,

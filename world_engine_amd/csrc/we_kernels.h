@@ -66,6 +66,7 @@ struct AttnParams {
   // measurement aid (null = off): every workgroup of the main kernel leaves its duration as
   // (shader-clock cycles, ticks of the constant 100 MHz counter) at [2 * linear workgroup id]
   uint64_t* clock_out;
+  int q_dma;            // 128-query workgroups fetch their Q tile by DMA (row offsets fit 32 bits)
 };
 
 // The merged q/k/v projection with the store's work as its epilogue (qkv_proj_store.hip).
@@ -94,5 +95,7 @@ hipError_t launch_attn_ring_f16_64(const AttnParams& p, int ksplit, hipStream_t 
 // fp32 caches: plain vector-ALU kernel, one pass, no context splitting
 hipError_t launch_attn_ring_f32(const AttnParams& p, int Dh, hipStream_t stream);
 hipError_t launch_attn_combine(const AttnParams& p, int Dh, int dtype, hipStream_t stream);
+// Measurement aid (stream_probe.hip): the 256-token-frame tile stream without the arithmetic.
+hipError_t launch_stream_probe(const void* src, int workgroups, int tiles, int share, hipStream_t stream);
 
 }  // namespace we

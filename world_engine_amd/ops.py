@@ -258,6 +258,18 @@ def attn_ring_static(q: Tensor, kv: Tensor, written: Tensor, t_pos: Tensor, L: i
     return out
 
 
+def stream_probe(buf: Tensor, workgroups: int, tiles: int, share: int = 1) -> None:
+    """Measurement aid (``we_stream_probe``): ``workgroups`` workgroups each stream ``tiles`` 16-KB
+    tiles of ``buf`` into LDS the way the attention kernel fetches K/V tiles at 256-token frames,
+    ``share`` workgroups per region, and compute nothing.  Time the launches from outside."""
+    dev = _need_device(buf)
+    if not buf.is_contiguous():
+        raise RuntimeError("buf must be contiguous")
+    code = _call(dev, _capi.lib().we_stream_probe, buf.data_ptr(), buf.numel() * buf.element_size(), workgroups, tiles,
+                 share, _stream_ptr(dev))
+    _capi.check(code, "we_stream_probe")
+
+
 def _build_extras(dtype, B, H, Hkv, T, Dh, qk_norm_eps, v1, v_lamb, gate, gate_x, gate_w):
     """``we_attn_extras`` for a call, or None.  Returns (pointer or None, object to keep alive)."""
     if not (qk_norm_eps or v1 is not None or gate is not None or gate_w is not None):
