@@ -83,11 +83,12 @@ AttnPlan plan_attn(int B, int H, int Hkv, int T, int64_t L, int n_splits, int va
     pl.n_splits = n_splits;
   } else if (wgs < 256) {
     // Never more workgroups than CUs (a second, nearly empty round costs a whole kernel's
-    // time); and when the context is cut four ways or more, fewer workgroups than CUs: the parts
-    // get longer, the partial results fewer, and the memory system, not the number of CUs, is
-    // what 256-token frames wait for (cfg1: 6 parts 25.1 us per frame-step, 8 parts 27.2; 24
-    // rings: 653 against 717).  Measured over 8 to 160 workgroups per call: the best count is
-    // about 240 workgroups for up to six parts and about 192 for more.
+    // time); and when the context is cut four ways or more, fewer workgroups than CUs: a part's
+    // fixed costs do not shrink with its length, the partial results grow with the number of
+    // parts, and the board clocks the kernel lower the more CUs are busy (cfg1: 6 parts 25.1 us
+    // per frame-step, 8 parts 27.2; 24 rings: 653 against 717).  Measured over 8 to 160
+    // workgroups per call: the best count is about 240 workgroups for up to six parts and about
+    // 192 for more.
     int64_t s = 256 / wgs;
     if (s >= 4) s = (wgs >= 40 ? 240 : 192) / wgs;
     if (s > max_s) s = max_s;
