@@ -73,6 +73,13 @@ def test_workspace_and_split_planning():
     for heads, want in ((24, 5), (40, 3), (48, 2), (80, 1)):
         assert lib.we_attn_auto_splits(1, heads, heads, 256, 128, 4096) == want, heads
     assert lib.we_attn_workspace_bytes(1, 16, 16, 256, 128, 4096, 0, 0) == s * 16 * 256 * (128 * 2 + 16)
+    # long contexts (32 slots and more) take about 240 workgroups; 32 heads are cut in four (all 256 CUs);
+    # beyond sixteen parts about 160 workgroups
+    assert lib.we_attn_auto_splits(1, 16, 16, 256, 128, 8192) == 7
+    assert lib.we_attn_auto_splits(1, 12, 12, 256, 128, 8192) == 10
+    assert lib.we_attn_auto_splits(1, 32, 32, 256, 128, 4096) == 4
+    assert lib.we_attn_auto_splits(1, 4, 4, 256, 128, 4096) == 20
+    assert lib.we_attn_auto_splits(1, 4, 4, 256, 128, 8192) == 20
     # 1024-token frames with 96 heads: 384 workgroups of 256 queries = 1.5 rounds of 256 CUs, so only
     # the last 32 of the 96 units (128 workgroups) are split in two
     assert lib.we_attn_auto_splits(4, 24, 24, 1024, 128, 8192) == 2

@@ -89,8 +89,14 @@ AttnPlan plan_attn(int B, int H, int Hkv, int T, int64_t L, int n_splits, int va
     // per frame-step, 8 parts 27.2; 24 rings: 653 against 717).  Measured over 8 to 160
     // workgroups per call: the best count is about 240 workgroups for up to six parts and about
     // 192 for more.
+    // Long contexts (32 slots of a 256-token frame and more) amortise the extra parts and the lower
+    // clock over longer loops: about 240 workgroups there too (cfg4: 7 parts 32.0 us per frame-step,
+    // 6 parts 32.8), and all 256 when that is exactly four parts (64 workgroups: 4 parts beat 3 by
+    // 2 to 7 %).
+    // Beyond sixteen parts every part's own cost weighs more: about 160 workgroups (4 heads: 20
+    // parts 21.2 to 27.2 us per frame-step over 16 to 64 slots, 24 parts 21.7 to 27.4).
     int64_t s = 256 / wgs;
-    if (s >= 4) s = (wgs >= 40 ? 240 : 192) / wgs;
+    if (s > 4) s = ((wgs >= 40 || (tiles >= 96 && 240 / wgs <= 16)) ? 240 : (192 / wgs > 16 ? 160 : 192)) / wgs;
     if (s > max_s) s = max_s;
     if (s > 64) s = 64;
     if (s < 1) s = 1;
