@@ -59,8 +59,9 @@ struct AttnPlan {
 //  * Shape: 256 queries per workgroup when that alone gives at least one workgroup per CU, else
 //    128 queries (two wavefronts share each query block and split every tile's keys).
 //  * Few workgroups (256-token frames): every unit is split into the same number of context
-//    parts - as many as fit the CUs in one round, three quarters of that from four parts on -
-//    but never fewer than two 64-key tiles per part.
+//    parts - as many as fit the CUs in one round up to four parts, then as many as give 160 to
+//    240 workgroups (more for long contexts, fewer for many parts) - but never fewer than two
+//    64-key tiles per part.
 //  * Many workgroups that do not divide into whole rounds of 256 CUs (e.g. 384): only the units
 //    of the last, partial round are split, so that round finishes in a fraction of the time.
 AttnPlan plan_attn(int B, int H, int Hkv, int T, int64_t L, int n_splits, int variant) {
