@@ -48,6 +48,7 @@
 #include "../../include/we_attn.h"
 
 #include <atomic>
+#include <type_traits>
 
 namespace we {
 
@@ -153,7 +154,7 @@ attn_ring_kernel(AttnParams p) {
   // below cannot go out before Q is back.  There the workgroup's 128 x Dh tile comes by DMA - 16
   // lanes per row, whole cache lines - into the V ring's slots 2 and 3, laid out and swizzled like
   // two K tiles, while the slot flags are on their way; the fragments are read from there once the
-  // first K tile is in, and slot 3 is zeroed afterwards.
+  // first K tile is in (the V stream's first request for those slots goes out after the next barrier).
   constexpr int Q_OFF = L::V_OFF + 2 * TILE_B;
   const bool q_dma = KSPLIT == 2 && p.q_dma != 0;
   frag_t qf[KS];
@@ -390,7 +391,10 @@ attn_ring_kernel(AttnParams p) {
   // nkeys: keys that exist in the block whose logits this step computes (32 = all, 0 = the block
   // lies past the end of the split)
   // (the K fragments at koff_c were requested by the previous step; the offset documents the call)
-  auto step = [&](auto /*koff_c*/, auto voff_c, auto nkoff_c, auto nvoff_c, int nkeys, auto&& mid) __attribute__((always_inline)) {
+  // first_c (128-query shape only): the workgroup's very first step has no previous block, so it
+  // skips the product and its V reads instead of multiplying a zeroed tile by zeros.
+  auto step = [&](auto /*koff_c*/, auto voff_c, auto nkoff_c, auto nvoff_c, int nkeys, auto&& mid, auto first_c) __attribute__((always_inline)) {
+    constexpr bool FIRST = decltype(first_c)::value;
     // (logits of a block past the end of the split are never consumed; a short tile's empty block
     // is masked after its products)
     // next own V fragment to request / next-step read pairs requested so far
@@ -433,7 +437,7 @@ attn_ring_kernel(AttnParams p) {
     for (int ks = 0; ks < KS; ++ks) {
       s_next = M::mma(__builtin_bit_cast(frag_t, kf[ks]), qf[ks], ks == 0 ? zero16 : s_next);
       // keep the read queue full without exceeding the 15 reads the counter can track
-      if (vnext < NV && ks <= 12 - KS) {
+      if (!FIRST && vnext < NV && ks <= 12 - KS) {
         read_v(voff_c, vnext);
         ++vnext;
         }
@@ -444,13 +448,15 @@ attn_ring_kernel(AttnParams p) {
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      if (vnext < NV) {  // reads 0..KS+2i-1 have completed: room for one more fragment
-        read_v(voff_c, vnext);
-        ++vnext;
+      if (!FIRST) {
+        if (vnext < NV) {  // reads 0..KS+2i-1 have completed: room for one more fragment
+          read_v(voff_c, vnext);
+          ++vnext;
         }
-      typedef unsigned int u32x4v __attribute__((ext_vector_type(4)));
-      const u32x4v a4 = __builtin_shufflevector(v0[i], v1[i], 0, 1, 2, 3);
-      o[i % DB] = M::mma(__builtin_bit_cast(frag_t, a4), p_prev[i / DB], o[i % DB]);
+        typedef unsigned int u32x4v __attribute__((ext_vector_type(4)));
+        const u32x4v a4 = __builtin_shufflevector(v0[i], v1[i], 0, 1, 2, 3);
+        o[i % DB] = M::mma(__builtin_bit_cast(frag_t, a4), p_prev[i / DB], o[i % DB]);
+      }
       if (i >= I0 && npair < NPAIR) next_pair();
       // VALU slices: the last exponentials; packing of the two 16-key halves and their row sums
       exp_slot(KS + i);
@@ -495,13 +501,13 @@ attn_ring_kernel(AttnParams p) {
   };
 
   if (ntile > 0) {
-    // zero V slot 3, which stands in for "tile -1", and P, so the first product adds zeros
-    auto zero_v3 = [&]() __attribute__((always_inline)) {
+    // 256-query shape: zero V slot 3, which stands in for "tile -1", and P, so that the first
+    // product adds zeros (the 128-query shape skips the product of its first step instead)
+    if (KSPLIT == 1) {
       const u32x4_t z = {0u, 0u, 0u, 0u};
       unsigned char* vz = smem + L::V_OFF + 3 * TILE_B;
       for (int i = tid; i < TILE_B / 16; i += 512) *reinterpret_cast<u32x4_t*>(vz + i * 16) = z;
-    };
-    if (!q_dma) zero_v3();  // (with the Q tile staged there: once its fragments have been read)
+    }
     {
       const u32x4_t z = {0u, 0u, 0u, 0u};
       p_prev[0] = __builtin_bit_cast(frag_t, z);
@@ -539,7 +545,7 @@ attn_ring_kernel(AttnParams p) {
       dma_v(o1, 1);
     }
     dma_wait<(KA + 1) * NDMA>();
-    __syncthreads();  // K(0) and the zeroed V slot (or the Q tile, requested long before K(0)) are in LDS
+    __syncthreads();  // K(0) and the zeroed V slot (128-query shape: the Q tile, requested long before K(0)) are in LDS
     if (KSPLIT == 2 && q_dma) {
       // row qb*32 + l32 of the tile, logical chunk 2*ks + hh: the K fragment's address arithmetic
       const int x = k_swz<DH>(l32);
@@ -566,18 +572,20 @@ attn_ring_kernel(AttnParams p) {
       }
       set_shift();
     }
-    if (KSPLIT == 2 && q_dma) {
-      __syncthreads();  // every wavefront has its Q fragments: the staging area becomes V slots again
-      zero_v3();
-    }
+    // (every wavefront has read its Q fragments before it passes the barrier below: the staging area
+    // becomes V slots again)
     dma_wait<2 * NDMA>();
     __syncthreads();  // everything but the last K and V tile issued so far has landed
     // first reads of the first step
-    if (KSPLIT == 1) prefetch(IntC<KB_B>(), IntC<3 * TILE_B + KB_B>());
-    else prefetch(IntC<TILE_B>(), IntC<3 * TILE_B>());
+    if (KSPLIT == 1) {
+      prefetch(IntC<KB_B>(), IntC<3 * TILE_B + KB_B>());
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) read_k(IntC<TILE_B>(), ks);
+    }
 
     // one tile iteration with compile-time ring positions (JM = j mod 4)
-    auto iteration = [&](int j, auto jm_c) __attribute__((always_inline)) {
+    auto iteration = [&](int j, auto jm_c, auto first_c) __attribute__((always_inline)) {
       constexpr int JM = decltype(jm_c)::value;
       auto issue_dma = [&]() __attribute__((always_inline)) {
         const uint32_t o = next_off();
@@ -592,16 +600,16 @@ attn_ring_kernel(AttnParams p) {
       if (KSPLIT == 1) {
         // block (j, 0) -> probabilities; logits of (j, 1); product of (j-1, 1)
         step(IntC<JM * TILE_B + KB_B>(), IntC<((JM + 3) % NST) * TILE_B + KB_B>(),
-             IntC<((JM + 1) % NST) * TILE_B>(), IntC<JM * TILE_B>(), block_keys(csub, 1), issue_dma);
+             IntC<((JM + 1) % NST) * TILE_B>(), IntC<JM * TILE_B>(), block_keys(csub, 1), issue_dma, std::false_type());
         // block (j, 1) -> probabilities; logits of (j+1, 0); product of (j, 0)
         step(IntC<((JM + 1) % NST) * TILE_B>(), IntC<JM * TILE_B>(),
              IntC<((JM + 1) % NST) * TILE_B + KB_B>(), IntC<JM * TILE_B + KB_B>(),
-             j + 1 < ntile ? block_keys(nsub, 0) : 0, nothing);
+             j + 1 < ntile ? block_keys(nsub, 0) : 0, nothing, std::false_type());
       } else {
         // block (j, hb) -> probabilities; logits of (j+1, hb); product of (j-1, hb)
         step(IntC<((JM + 1) % NST) * TILE_B>(), IntC<((JM + 3) % NST) * TILE_B>(),
              IntC<((JM + 2) % NST) * TILE_B>(), IntC<JM * TILE_B>(),
-             j + 1 < ntile ? block_keys(nsub, __builtin_amdgcn_readfirstlane(hb)) : 0, issue_dma);
+             j + 1 < ntile ? block_keys(nsub, __builtin_amdgcn_readfirstlane(hb)) : 0, issue_dma, first_c);
       }
       csub = nsub;
       dma_wait<2 * NDMA>();  // all but this iteration's two tiles have landed (this wavefront's part)
@@ -615,15 +623,25 @@ attn_ring_kernel(AttnParams p) {
     };
 
     int j = 0;
-    for (; j + 4 <= ntile; j += 4) {
-      iteration(j, IntC<0>());
-      iteration(j + 1, IntC<1>());
-      iteration(j + 2, IntC<2>());
-      iteration(j + 3, IntC<3>());
+    const std::false_type not_first;
+    if (KSPLIT == 2) {
+      // the first tile's step has no product to do: peeled, with the three iterations that bring
+      // the ring position back to zero
+      iteration(0, IntC<0>(), std::true_type());
+      j = 1;
+      if (j < ntile) { iteration(j, IntC<1>(), not_first); ++j; }
+      if (j < ntile) { iteration(j, IntC<2>(), not_first); ++j; }
+      if (j < ntile) { iteration(j, IntC<3>(), not_first); ++j; }
     }
-    if (j < ntile) { iteration(j, IntC<0>()); ++j; }
-    if (j < ntile) { iteration(j, IntC<1>()); ++j; }
-    if (j < ntile) { iteration(j, IntC<2>()); ++j; }
+    for (; j + 4 <= ntile; j += 4) {
+      iteration(j, IntC<0>(), not_first);
+      iteration(j + 1, IntC<1>(), not_first);
+      iteration(j + 2, IntC<2>(), not_first);
+      iteration(j + 3, IntC<3>(), not_first);
+    }
+    if (j < ntile) { iteration(j, IntC<0>(), not_first); ++j; }
+    if (j < ntile) { iteration(j, IntC<1>(), not_first); ++j; }
+    if (j < ntile) { iteration(j, IntC<2>(), not_first); ++j; }
 
     // product of the last block: (ntile-1, 1) for full-tile wavefronts, (ntile-1, hb) otherwise
     {
