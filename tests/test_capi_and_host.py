@@ -221,6 +221,19 @@ def test_one_call_entry_point_validates_both_halves():
     assert lib.we_rope_kv_attn_fwd(*args(extras=ctypes.byref(ex))) == -2
 
 
+def test_stream_probe_validates_before_launching():
+    """The tile-stream measurement aid refuses bad arguments with a status code (no GPU needed)."""
+    lib = _capi.lib()
+    fake = ctypes.c_void_p(4096)
+    region = 23 * 16384
+    assert lib.we_stream_probe(None, 96 * region, 192, 23, 2, None) == -1            # null buffer
+    assert lib.we_stream_probe(fake, 96 * region, 100, 23, 2, None) == -2            # workgroups not a multiple of 8
+    assert lib.we_stream_probe(fake, 96 * region, 192, 0, 2, None) == -2             # no tiles
+    assert lib.we_stream_probe(fake, 96 * region, 192, 23, 5, None) == -2            # 24 workgroups per XCD do not share in fives
+    assert lib.we_stream_probe(ctypes.c_void_p(4100), 96 * region, 192, 23, 2, None) == -4   # misaligned
+    assert lib.we_stream_probe(fake, 96 * region - 1, 192, 23, 2, None) == -5        # buffer does not cover the regions
+
+
 def test_projection_entry_points_validate_before_launching():
     """we_qkv_rope_kv_store / we_qkv_rope_kv_attn_fwd refuse bad operands with a status code and
     launch nothing (no GPU is needed to see that)."""
