@@ -467,6 +467,48 @@ def test_ring_attn_module_matches_cpu_composition(gpu_device, fuse):
         assert torch.equal(cache.layers[0].written.cpu(), ocache.layers[0].written)
 
 
+def test_calls_from_a_worker_thread(gpu_device):
+    """The reference generates frames from a worker thread (asyncio.to_thread(engine.gen_frame, ...),
+    examples/simple_client.py:23-25) and from its own stream.  The library launches on the calling
+    thread's current stream and keeps no per-thread state: frames stepped alternately by the main
+    thread and by a worker thread on a side stream must leave the same cache state and outputs as
+    the oracle."""
+    import threading
+    p = Pair(gpu_device, torch.bfloat16, B=1, H=4, Hkv=2, T=128, Dh=128, n_slots=3, cfg_id=28)
+    p.set_frozen(False)
+    side = torch.cuda.Stream(device=gpu_device)
+    results, errors = {}, []
+
+    def one_frame(t, use_side):
+        try:
+            q, k, v, pos = p.inputs(t)
+            if use_side:
+                side.wait_stream(torch.cuda.default_stream(gpu_device))
+                with torch.cuda.stream(side):
+                    (q_o, k_all, v_all, mask), (q_h, ring) = p.store(q, k, v, pos)
+                    out = p.attend(q_h, ring)
+                side.synchronize()
+            else:
+                (q_o, k_all, v_all, mask), (q_h, ring) = p.store(q, k, v, pos)
+                out = p.attend(q_h, ring)
+                torch.cuda.synchronize()
+            results[t] = (out, ro.attention_fp32(q_o, k_all, v_all, mask))
+        except Exception as e:          # noqa: BLE001 - re-raised in the main thread
+            errors.append((t, e))
+
+    for t in range(6):
+        _say(f"worker thread frame {t}")
+        if t % 2:
+            th = threading.Thread(target=one_frame, args=(t, True))
+            th.start()
+            th.join()
+        else:
+            one_frame(t, False)
+        assert not errors, errors
+        p.assert_state_equal(what=f"t={t}")
+        assert_attn_close(*results[t], f"t={t}")
+
+
 def test_hip_graph_replay_matches_eager(gpu_device):
     """One frame step (store + attention) captured in a HIP graph and replayed for successive
     frames by updating only device tensors; every replay must equal the eager result."""
