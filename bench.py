@@ -65,6 +65,17 @@ def algorithmic_work(c, n_vis):
     return flops, byts
 
 
+def store_work(c, persisting):
+    """Algorithmic bytes of one RoPE + ring-store call (the store kernel is HBM-bound): q, k and v
+    of the frame read once; RoPE(q) and the tail's K and V rows written once, the ring slot's K and
+    V rows as well on a persisting call; the position ids and the cos / sin rows of the frame's
+    tokens read once per batch row."""
+    e, B, H, Hkv, T, Dh = 2.0, c["B"], c["H"], c["Hkv"], c["T"], c["Dh"]
+    read = e * B * T * Dh * (H + 2 * Hkv) + B * T * (3 * 8 + 2 * 4 * Dh / 2)
+    written = e * B * T * Dh * (H + 2 * Hkv * (2 if persisting else 1))
+    return read + written
+
+
 def schedule_plan(c, steps, warmup, cpu_window=8):
     """Frame arithmetic of one configuration's run, in one place so that it can be checked without
     a GPU.  Step s of the schedule belongs to frame s // subs (subs = attention calls per frame).
@@ -166,9 +177,12 @@ def run_gpu(cfg_id, c, args, torch, ro, wea, ops):
     nf = plan["attn_frame"] + 1
     t_pos_all = torch.arange(nf, dtype=torch.long)[:, None, None].expand(nf, B, T).contiguous().to(dev)
 
-    n_splits = args.n_splits or ops.attn_auto_splits(B, H, Hkv, T, Dh, L)
-    ws = torch.empty(max(ops.attn_workspace_bytes(B, H, Hkv, T, Dh, L, args.n_splits, args.q_tile), 16),
-                     dtype=torch.uint8, device=dev)
+    from world_engine_amd import _capi
+    q_tile = args.q_tile | (_capi.WE_SPLIT_TWO_PASS if args.two_pass else 0)
+    ops.init(dev)
+    lib_plan = ops.attn_plan(B, H, Hkv, T, Dh, L, args.n_splits, args.q_tile, xcd_merge=None, two_pass=args.two_pass)
+    n_splits = lib_plan["n_splits"]
+    ws = ops.new_workspace(max(ops.attn_workspace_bytes(B, H, Hkv, T, Dh, L, args.n_splits, q_tile), 16), dev)
     out = torch.empty((B, T, H, Dh), dtype=dtype, device=dev).transpose(1, 2)
 
     def one_step(step_idx):
@@ -183,10 +197,10 @@ def run_gpu(cfg_id, c, args, torch, ro, wea, ops):
                 q_rot = ops.rope_kv_store(q, k, v, pos, rope.cos, rope.sin, rope.height, rope.width,
                                           layer.kv, layer.written, layer.L, 1, frozen)
                 ops.attn_ring(q_rot, layer.kv, layer.written, pos["t_pos"], layer.L, 1, n_splits=args.n_splits,
-                              q_tile=args.q_tile, out=out, workspace=ws)
+                              q_tile=q_tile, out=out, workspace=ws)
             else:
                 ops.rope_kv_attn(q, k, v, pos, rope.cos, rope.sin, rope.height, rope.width, layer.kv,
-                                 layer.written, layer.L, 1, frozen, n_splits=args.n_splits, q_tile=args.q_tile,
+                                 layer.written, layer.L, 1, frozen, n_splits=args.n_splits, q_tile=q_tile,
                                  out=out, workspace=ws)
 
     if args.calibrate_copy:
@@ -242,7 +256,7 @@ def run_gpu(cfg_id, c, args, torch, ro, wea, ops):
 
     def attn_only():
         ops.attn_ring(q_rot, layer0.kv, layer0.written, pos["t_pos"], layer0.L, 1, n_splits=args.n_splits,
-                      q_tile=args.q_tile, out=out, workspace=ws)
+                      q_tile=q_tile, out=out, workspace=ws)
 
     for _ in range(5):
         attn_only()
@@ -287,12 +301,56 @@ def run_gpu(cfg_id, c, args, torch, ro, wea, ops):
                 "frac": round(tflops / PEAK_BF16_TFLOPS, 4), "traffic": None}
     if not (args.n_splits or args.q_tile):
         roof["traffic"], roof["traffic_source"] = read_traffic(cfg_id)
-    roof.update({"kernel": "attn_ring_kernel" + (" + attn_combine_kernel" if n_splits > 1 else ""),
+    roof.update({"kernel": "attn_ring_kernel" + (" + attn_combine_kernel" if n_splits > 1 and not lib_plan["merge_in_kernel"] else ""),
+                 "split_parts_merged": ("nothing split" if n_splits == 1 else
+                                        "inside attn_ring_kernel (last workgroup of a query tile, through its XCD's L2)"
+                                        if lib_plan["merge_in_kernel"] else "by attn_combine_kernel"),
+                 "workgroups": lib_plan["workgroups"], "compute_units": lib_plan["compute_units"],
                  "us_per_launch": round(attn_us, 3), "us_per_launch_p10": round(ast["p10"], 3),
                  "us_per_launch_p90": round(ast["p90"], 3), "launches_per_sample": iters,
                  "algorithmic_bytes": byts, "algorithmic_flops": flops, "n_splits": n_splits,
                  "tflops": round(tflops, 2), "algorithmic_gbps": round(gbps, 1)})
     log(f"[bench] attention call: {attn_us:.2f} us -> {tflops:.1f} TFLOP/s, {gbps:.0f} GB/s algorithmic")
+
+    # ---- the store kernel alone against its own (HBM) roofline: a graph of persisting store-only calls ----
+    store_roof = None
+    if not args.eager:
+        q0, k0, v0 = inputs[0]
+
+        def store_only():
+            ops.rope_kv_store(q0, k0, v0, pos, rope.cos, rope.sin, rope.height, rope.width, layer0.kv, layer0.written,
+                              layer0.L, 1, False)
+
+        for _ in range(3):
+            store_only()
+        torch.cuda.synchronize()
+        g3 = torch.cuda.CUDAGraph()
+        side3 = torch.cuda.Stream()
+        side3.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.graph(g3, stream=side3):
+            for _ in range(iters):
+                store_only()
+        torch.cuda.synchronize()
+        g3.replay()
+        torch.cuda.synchronize()
+        st_samples = []
+        for _ in range(SAMPLES):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            g3.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            st_samples.append(e0.elapsed_time(e1) * 1e3 / iters)
+        sst = spread(st_samples)
+        sbytes = store_work(c, True)
+        sgbps = sbytes / (sst["median"] * 1e-6) / 1e9
+        store_roof = {"kernel": "rope_kv_store_kernel", "bound": "hbm", "achieved": round(sgbps, 1), "peak": PEAK_HBM_GBPS,
+                      "unit": "GB/s", "frac": round(sgbps / PEAK_HBM_GBPS, 4), "us_per_launch": round(sst["median"], 3),
+                      "us_per_launch_p10": round(sst["p10"], 3), "us_per_launch_p90": round(sst["p90"], 3),
+                      "launches_per_sample": iters, "algorithmic_bytes": sbytes,
+                      "what": "persisting call: q, k, v read; RoPE(q), tail rows and ring-slot rows written"}
+        log(f"[bench] store call: {sst['median']:.2f} us -> {sgbps:.0f} GB/s algorithmic")
+        del g3
 
     # ---- shader clock inside the main kernel: cycles against the constant 100 MHz counter, per workgroup ----
     if not args.eager:
@@ -300,7 +358,7 @@ def run_gpu(cfg_id, c, args, torch, ro, wea, ops):
             clocks = torch.zeros(2 * 65536, dtype=torch.int64, device=dev)
             for _ in range(60):                       # back to back, so the board sits at its sustained clock
                 ops.attn_ring(q_rot, layer0.kv, layer0.written, pos["t_pos"], layer0.L, 1, n_splits=args.n_splits,
-                              q_tile=args.q_tile, out=out, workspace=ws, clocks=clocks)
+                              q_tile=q_tile, out=out, workspace=ws, clocks=clocks)
             torch.cuda.synchronize()
             ck = clocks.view(-1, 2).cpu()
             ck = ck[ck[:, 1] > 0].double()
@@ -322,7 +380,7 @@ def run_gpu(cfg_id, c, args, torch, ro, wea, ops):
            "us_per_step_p90": round(st["p90"], 3), "samples": st["samples"], "replays_per_sample": reps,
            "us_per_layer_step": round(st["median"] / layers, 3), "layers": layers, "calls_per_frame": subs,
            "launch": "eager" if args.eager else "hip_graph", "n_splits": n_splits, "q_tile": args.q_tile or "auto",
-           "roofline": roof}
+           "roofline": roof, "store_roofline": store_roof}
     del cache, ws, out, inputs, t_pos_all
     torch.cuda.empty_cache()
     return res
@@ -577,6 +635,9 @@ def main():
                     help="only the projection + store measurement (with --calibrate-copy: preceded by the copy kernels "
                          "of known traffic, for a counter run)")
     ap.add_argument("--no-peaks", action="store_true", help="skip the measured GEMM / copy rates of this box")
+    ap.add_argument("--two-pass", action="store_true",
+                    help="merge split-context parts with the second kernel even where the main kernel would do it "
+                         "itself (WE_SPLIT_TWO_PASS; for same-box comparisons)")
     ap.add_argument("--two-calls", action="store_true",
                     help="we_rope_kv_store + we_attn_ring_fwd instead of the one-call we_rope_kv_attn_fwd")
     ap.add_argument("--attn-iters", type=int, default=200, help="attention-only launches for the roofline timing")
@@ -673,7 +734,8 @@ def main():
                       f"{args.steps}-step HIP graph between device synchronisations"})
         result.update({"p10": h["us_per_step_p10"], "p90": h["us_per_step_p90"],
                        "us_per_layer_step": h["us_per_layer_step"], "attn_tflops": h["roofline"]["tflops"],
-                       "attn_algorithmic_gbps": h["roofline"]["algorithmic_gbps"], "roofline": h["roofline"]})
+                       "attn_algorithmic_gbps": h["roofline"]["algorithmic_gbps"], "roofline": h["roofline"],
+                       "store_roofline": h.get("store_roofline")})
     result.update(extras)
 
     # ---- CPU baselines: the oracle's restatement of the reference path on the host cores ----

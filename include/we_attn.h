@@ -8,11 +8,12 @@
  *   kv_cache.upsert(k, v, pos_ids, layer) src/model/kv_cache.py:104-154, :191-193
  *   flex_attention(q, k, v, block_mask)   src/model/attn.py:116, src/patch_model.py:133
  *
- * world_engine has no native code: these are the calls a binding would replace with the two
+ * world_engine has no native code: these are the calls a binding would replace with the
  * entry points below.  All pointers are DEVICE pointers owned by the caller.  Every call only
- * enqueues work on `stream`; it never synchronises, never allocates and keeps no mutable
- * global state (beyond raising each kernel's dynamic-LDS limit once), so it is re-entrant and
- * capturable into a HIP graph.  The frame index that
+ * enqueues work on `stream`; it never allocates and - after the one-time set-up of the device it
+ * runs on, see we_init - never synchronises, so it is re-entrant and capturable into a HIP graph.
+ * The only state the library keeps is what that set-up found out about each device (read-only
+ * afterwards).  The frame index that
  * selects the ring slot is read by the kernels from device memory (`t_pos[0]`), exactly as the
  * reference derives it from a device tensor (src/model/kv_cache.py:126), so no host value of
  * it is ever needed.
@@ -42,17 +43,37 @@ extern "C" {
 #define WE_ERR_WORKSPACE (-5)     /* split-context workspace missing or too small */
 #define WE_ERR_LAUNCH (-6)        /* the HIP runtime refused the launch */
 #define WE_ERR_SCRATCH_LIMIT (-7) /* we_attn_ring_fwd_static: sizes need more scratch than WE_STATIC_SCRATCH_BYTES */
+#define WE_ERR_NOT_READY (-8)     /* first call on a device made under stream capture: call we_init() beforehand */
 
 #define WE_MAX_SLOTS 256 /* maximum number of ring slots L / T */
 
 /* size of the library's own split-context scratch buffer (see we_attn_ring_fwd_static) */
 #define WE_STATIC_SCRATCH_BYTES (32u << 20)
 
+/* leading bytes of a split-context workspace that hold arrival counters (see we_attn_ring_fwd) */
+#define WE_WS_COUNTER_BYTES 16384
+
+/* OR into q_tile: merge split-context parts with the second kernel even where the main kernel
+ * could do it itself (same results, bit for bit; for comparisons) */
+#define WE_SPLIT_TWO_PASS 0x10000
+
 /* Library version: major*10000 + minor*100 + patch. */
 int we_version(void);
 
 /* Static description of a WE_ERR_* code. */
 const char* we_error_string(int code);
+
+/*
+ * One-time set-up of the CURRENT device (hipSetDevice), without a counterpart in the reference:
+ * raises the kernels' dynamic-LDS limits, looks up the static scratch buffer's address and runs a
+ * small probe launch on the null stream that checks how the hardware deals workgroups to the
+ * XCDs (the in-kernel merge of split-context parts is only used where workgroup id % 8 names the
+ * XCD).  Synchronises the device once; idempotent and thread-safe.  Every entry point that
+ * launches does the same implicitly on its first call on a device - except when its stream is
+ * being captured, where it returns WE_ERR_NOT_READY instead: callers that capture graphs call
+ * we_init() (or make one ordinary call) on the device first.
+ */
+int we_init(void);
 
 /*
  * Fused RoPE + ring-slot K/V store for one frame.
@@ -116,11 +137,25 @@ int32_t we_attn_auto_splits(int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_
 
 /*
  * Bytes of split-context workspace we_attn_ring_fwd needs for these sizes and the given n_splits /
- * q_tile arguments (0 when nothing is split).  Sizing helper without a counterpart in the
- * reference.
+ * q_tile arguments (0 when nothing is split; otherwise WE_WS_COUNTER_BYTES + the partial
+ * results).  Depends on the compute-unit count of the current device (256 when there is none to
+ * ask).  Sizing helper without a counterpart in the reference.
  */
 size_t we_attn_workspace_bytes(int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L,
                                int32_t n_splits, int32_t q_tile);
+
+/*
+ * What the library would do with an attention call of these sizes (inspection helper without a
+ * counterpart in the reference; launches nothing): plan[0] = queries per workgroup, [1] = context
+ * parts of the units that are split, [2] = leading (batch, kv head) units left whole, [3] = 1 when
+ * the main kernel merges the parts itself (0: second kernel), [4] = workgroups of the main launch,
+ * [5] = compute units planned for.  compute_units = 0 asks the current device (256 without one);
+ * xcd_merge: 1 / 0 = assume that the device passed / failed we_init's XCD check, -1 = use what the
+ * current device's set-up found (runs it if need be, see we_init).
+ */
+#define WE_PLAN_FIELDS 6
+int we_attn_plan(int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L, int32_t n_splits,
+                 int32_t q_tile, int32_t compute_units, int32_t xcd_merge, int32_t plan[WE_PLAN_FIELDS]);
 
 /*
  * Frame-block-causal attention of one frame's queries over the ring buffer.
@@ -137,13 +172,23 @@ size_t we_attn_workspace_bytes(int32_t B, int32_t H, int32_t Hkv, int32_t T, int
  *   kv, written, t_pos   as in we_rope_kv_store, after that call for the same frame.
  *   out  [B, H, T, Dh]   element strides out_strides = {batch, head, token}; Dh contiguous.
  *   workspace            device scratch of at least we_attn_workspace_bytes(...) bytes for the
- *                        same sizes, n_splits and q_tile; may be NULL when that is 0.
+ *                        same sizes, n_splits and q_tile; may be NULL when that is 0.  Its first
+ *                        WE_WS_COUNTER_BYTES bytes hold arrival counters: they must be ZERO when
+ *                        the buffer is first handed to the library, and every call leaves them
+ *                        zero again (so a buffer is cleared once, when it is allocated, and can be
+ *                        reused by calls of any sizes that follow each other on a stream; calls
+ *                        that overlap in time need a workspace each).  The rest may hold anything.
  *   n_splits             0 = choose automatically (small grids: every (batch, kv head) unit is
- *                        split so that all CUs have work; grids that leave a partial last round
+ *                        split so that most CUs have work; grids that leave a partial last round
  *                        of workgroups: only that round's units are split); 1 = single pass;
  *                        2..64 = split the visible context of every unit into that many parts.
- *                        Split parts are combined by a second kernel.
- *   q_tile               queries per workgroup: 0 = choose automatically, or 128 / 256.
+ *                        The parts are merged by the main kernel itself - by whichever workgroup
+ *                        of a query tile finishes last, through the L2 of the XCD that all parts
+ *                        of a unit are placed on - when the device passed we_init's XCD check and
+ *                        both the split and the unsplit unit counts are multiples of 8; otherwise
+ *                        by a second kernel.  Both routes give the same bits.
+ *   q_tile               queries per workgroup: 0 = choose automatically, or 128 / 256;
+ *                        optionally | WE_SPLIT_TWO_PASS.
  *   scale                softmax scale (> 0); the reference uses 1/sqrt(Dh).
  *
  * Requirements: dtype bf16 or f16 (MFMA kernel) or f32 (plain one-pass kernel on the vector
@@ -160,51 +205,22 @@ int we_attn_ring_fwd(const void* q, const int64_t q_strides[3],
                      int32_t dtype, void* stream);
 
 /*
- * Measurement aid without a counterpart in the reference: we_attn_ring_fwd that also records how
- * long every workgroup of the main kernel ran, on two clocks.  clocks[2 * w] receives workgroup
- * w's duration in shader-clock cycles, clocks[2 * w + 1] the same interval in ticks of the
- * device's constant 100 MHz counter, w being the linear workgroup id of the launch; their ratio
- * is the shader clock the kernel actually ran at (boards lower it under their power limit).
- * clocks_len = number of uint64 elements available; at least 2 * (workgroups of the launch) or
- * WE_ERR_WORKSPACE is returned; entries of workgroups that own no work stay untouched (zero them
- * beforehand).  bf16 / f16 only.  Everything else as we_attn_ring_fwd.
- */
-int we_attn_ring_fwd_clocked(const void* q, const int64_t q_strides[3],
-                             const void* kv, const uint8_t* written, const int64_t* t_pos,
-                             void* out, const int64_t out_strides[3],
-                             void* workspace, size_t workspace_bytes,
-                             int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L,
-                             int32_t dilation, float scale, int32_t n_splits, int32_t q_tile,
-                             int32_t dtype, uint64_t* clocks, size_t clocks_len, void* stream);
-
-/*
- * Measurement aid without a counterpart in the reference: the attention kernel's way of fetching
- * K and V tiles at 256-token frames with the arithmetic taken away.  `workgroups` workgroups (one
- * per CU, a multiple of 8: workgroup id % 8 is the XCD) each stream `tiles` 16-KB tiles of one
- * contiguous region of `buf` into LDS by DMA, three tiles in flight, one barrier per tile;
- * `share` consecutive workgroups of an XCD walk the same region (the query tiles and grouped heads
- * of one K/V stream).  Region r starts at byte r * tiles * 16384; buf_bytes must cover the
- * workgroups / share regions (WE_ERR_WORKSPACE otherwise).  Nothing is written.  The duration of a
- * launch is the floor for a kernel of this shape, whatever it computes.
- */
-int we_stream_probe(const void* buf, size_t buf_bytes, int32_t workgroups, int32_t tiles, int32_t share,
-                    void* stream);
-
-/*
  * we_attn_ring_fwd for callers that cannot allocate device memory, not even a workspace: code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
  * counterpart in the reference (whose attention call allocates through torch as it pleases).
  * Arguments, requirements and results are those of we_attn_ring_fwd, bit for bit, without the
  * workspace pair: the split-context partial results go to a buffer of WE_STATIC_SCRATCH_BYTES that
  * is part of the library's device image (every GPU the library runs on holds one copy until the
- * process ends; its address is looked up once per device, on the first call made with that
- * device current).  Sizes whose we_attn_workspace_bytes(...) exceeds WE_STATIC_SCRATCH_BYTES are
+ * process ends; its address is looked up once per device by that device's set-up, see we_init:
+ * under stream capture the device must have been set up beforehand).  Sizes whose
+ * we_attn_workspace_bytes(...) exceeds WE_STATIC_SCRATCH_BYTES are
  * rejected with WE_ERR_SCRATCH_LIMIT and nothing is launched.  The call itself performs no
  * hipMalloc / hipFree and calls no allocating library routine.
  * All calls on one GPU share that GPU's buffer: calls that overlap in time on one GPU (different
  * streams, or parallel branches of one graph) race on it; calls that follow each other on a
- * stream do not.  Nothing in the buffer has to start at zero (every partial row a call reads was
- * written by that call's first kernel).
+ * stream do not.  The buffer's arrival counters are zero when the image is loaded and every call
+ * leaves them zero; nothing else in it has to start at any value (every partial row a call reads
+ * was written by that call).
  */
 int we_attn_ring_fwd_static(const void* q, const int64_t q_strides[3],
                             const void* kv, const uint8_t* written, const int64_t* t_pos,

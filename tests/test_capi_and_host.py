@@ -15,22 +15,42 @@ from world_engine_amd import _capi, ops
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def _declared_symbols():
-    text = open(os.path.join(ROOT, "include", "we_attn.h")).read()
+def _declared_symbols(header="we_attn.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(we_[a-z0-9_]+)\s*\(", text)))
 
 
+def _exported(path):
+    import subprocess
+    out = subprocess.run(["nm", "-D", "--defined-only", path], capture_output=True, text=True, check=True).stdout
+    return {line.split()[-1] for line in out.splitlines() if " T " in line and line.split()[-1].startswith("we_")}
+
+
 def test_library_exports_every_declared_symbol():
     names = _declared_symbols()
-    assert {"we_version", "we_error_string", "we_rope_kv_store", "we_rope_apply", "we_attn_auto_splits",
-            "we_attn_workspace_bytes", "we_attn_ring_fwd"} <= set(names)
+    assert {"we_version", "we_error_string", "we_init", "we_rope_kv_store", "we_rope_apply", "we_attn_auto_splits",
+            "we_attn_workspace_bytes", "we_attn_plan", "we_attn_ring_fwd"} <= set(names)
     assert set(names) == set(_capi.SIGNATURES), "ctypes signatures and header disagree"
     lib = _capi.lib()
     for n in names:
         assert hasattr(lib, n), f"{n} not exported"
     assert lib.we_version() >= 100
     assert lib.we_error_string(0) == b"ok" and b"unknown" in lib.we_error_string(-99)
+    # the product library is the drop-in surface and nothing else: no measurement entry points
+    assert _exported(_capi.LIB_PATH) == set(names)
+
+
+def test_measurement_library_exports_both_headers():
+    """libwe_probe.so (benchmark and probe tests only) carries the entry points of
+    include/we_attn_probe.h on top of the product's."""
+    probe_names = _declared_symbols("we_attn_probe.h")
+    assert set(probe_names) == set(_capi.PROBE_SIGNATURES) == {"we_attn_ring_fwd_clocked", "we_stream_probe"}
+    plib = _capi.probe_lib()
+    for n in probe_names + _declared_symbols():
+        assert hasattr(plib, n), f"{n} not exported by the measurement library"
+    assert _exported(_capi.PROBE_LIB_PATH) == set(probe_names) | set(_declared_symbols())
+    assert plib.we_version() == _capi.lib().we_version()
 
 
 def test_validation_codes_without_gpu():
@@ -65,14 +85,16 @@ def test_validation_codes_without_gpu():
 def test_workspace_and_split_planning():
     lib = _capi.lib()
     assert lib.we_attn_workspace_bytes(1, 16, 16, 256, 128, 4096, 1, 0) == 0
-    assert lib.we_attn_workspace_bytes(1, 16, 16, 256, 128, 4096, 4, 0) == 4 * 16 * 256 * (128 * 2 + 16)
+    hdr = _capi.WE_WS_COUNTER_BYTES      # arrival counters at the start of every split-context workspace
+    assert lib.we_attn_workspace_bytes(1, 16, 16, 256, 128, 4096, 4, 0) == hdr + 4 * 16 * 256 * (128 * 2 + 16)
+    assert lib.we_attn_workspace_bytes(1, 16, 16, 256, 128, 4096, 4, _capi.WE_SPLIT_TWO_PASS) == hdr + 4 * 16 * 256 * (128 * 2 + 16)
     # 256-token frames: every unit is split, into three quarters of the parts that would give every CU a workgroup
     s = lib.we_attn_auto_splits(1, 16, 16, 256, 128, 4096)
     assert s == 6
     # ... and the workgroups of a call never outnumber the 256 CUs: 48, 80, 96, 160 unsplit workgroups
     for heads, want in ((24, 5), (40, 3), (48, 2), (80, 1)):
         assert lib.we_attn_auto_splits(1, heads, heads, 256, 128, 4096) == want, heads
-    assert lib.we_attn_workspace_bytes(1, 16, 16, 256, 128, 4096, 0, 0) == s * 16 * 256 * (128 * 2 + 16)
+    assert lib.we_attn_workspace_bytes(1, 16, 16, 256, 128, 4096, 0, 0) == hdr + s * 16 * 256 * (128 * 2 + 16)
     # long contexts (32 slots and more) take about 240 workgroups; 32 heads are cut in four (all 256 CUs);
     # beyond sixteen parts about 160 workgroups
     assert lib.we_attn_auto_splits(1, 16, 16, 256, 128, 8192) == 7
@@ -83,12 +105,53 @@ def test_workspace_and_split_planning():
     # 1024-token frames with 96 heads: 384 workgroups of 256 queries = 1.5 rounds of 256 CUs, so only
     # the last 32 of the 96 units (128 workgroups) are split in two
     assert lib.we_attn_auto_splits(4, 24, 24, 1024, 128, 8192) == 2
-    assert lib.we_attn_workspace_bytes(4, 24, 24, 1024, 128, 8192, 0, 0) == 2 * 32 * 1024 * (128 * 2 + 16)
+    assert lib.we_attn_workspace_bytes(4, 24, 24, 1024, 128, 8192, 0, 0) == hdr + 2 * 32 * 1024 * (128 * 2 + 16)
     # whole rounds: nothing to split
     assert lib.we_attn_auto_splits(4, 32, 32, 1024, 128, 8192) == 1
     assert lib.we_attn_workspace_bytes(4, 32, 32, 1024, 128, 8192, 0, 0) == 0
     # never more splits than half the 64-key tiles of the context
     assert lib.we_attn_auto_splits(1, 1, 1, 64, 64, 128) <= 1
+
+
+def test_plan_reports_the_in_kernel_merge():
+    """16 units of a 256-token frame (benchmark configurations 1, 2 and 4) and the 32 tail units of
+    configuration 3 are merged in the kernel; unit counts that are not multiples of 8, a device
+    that did not pass the XCD check and the two-pass flag take the second kernel."""
+    assert ops.attn_plan(1, 16, 16, 256, 128, 4096, compute_units=256) == {
+        "q_tile": 128, "n_splits": 6, "units_whole": 0, "merge_in_kernel": True, "workgroups": 192, "compute_units": 256}
+    assert ops.attn_plan(1, 16, 16, 256, 128, 8192, compute_units=256)["merge_in_kernel"]
+    p3 = ops.attn_plan(4, 24, 24, 1024, 128, 8192, compute_units=256)
+    assert (p3["q_tile"], p3["n_splits"], p3["units_whole"], p3["merge_in_kernel"], p3["workgroups"]) == (256, 2, 64, True, 512)
+    assert not ops.attn_plan(1, 12, 12, 256, 128, 4096, compute_units=256)["merge_in_kernel"]
+    assert not ops.attn_plan(1, 16, 16, 256, 128, 4096, compute_units=256, xcd_merge=False)["merge_in_kernel"]
+    assert not ops.attn_plan(1, 16, 16, 256, 128, 4096, compute_units=256, two_pass=True)["merge_in_kernel"]
+
+
+def test_planner_over_other_shapes_and_cu_counts():
+    """Invariants of the split planner over shapes and parts other than the benchmark's: a split
+    call never launches more workgroups than there are CUs, every part keeps at least two 64-key
+    tiles, unsplit calls stay unsplit, and the counts scale with the CU count."""
+    for cus in (64, 104, 228, 256, 304):
+        for B, H, Hkv, T, n_slots in ((1, 4, 4, 256, 16), (1, 12, 4, 256, 24), (2, 8, 8, 128, 8), (1, 40, 40, 256, 32),
+                                      (1, 6, 2, 64, 3), (3, 5, 5, 192, 12), (1, 16, 16, 256, 64), (1, 2, 2, 512, 4)):
+            pl = ops.attn_plan(B, H, Hkv, T, 128, n_slots * T, compute_units=cus)
+            unsplit = B * H * -(-T // pl["q_tile"])
+            tiles = n_slots * T // 64
+            assert pl["compute_units"] == cus and pl["n_splits"] >= 1
+            if pl["n_splits"] > 1 and pl["units_whole"] == 0:
+                assert pl["workgroups"] <= cus, (cus, B, H, T, n_slots, pl)
+                assert pl["workgroups"] == unsplit * pl["n_splits"]
+                assert tiles // pl["n_splits"] >= 2, (cus, B, H, T, n_slots, pl)
+                assert pl["workgroups"] * 2 > cus or pl["n_splits"] == max(1, tiles // 2), "split calls use most of the chip"
+            if unsplit >= cus and unsplit % cus == 0:
+                assert pl["n_splits"] == 1
+            if pl["merge_in_kernel"]:
+                assert pl["units_whole"] % 8 == 0 and (B * Hkv - pl["units_whole"]) % 8 == 0
+    # the benchmark's 16-head call on half and on twice the CUs
+    assert ops.attn_plan(1, 16, 16, 256, 128, 4096, compute_units=128)["n_splits"] == 4
+    assert ops.attn_plan(1, 16, 16, 256, 128, 4096, compute_units=512)["n_splits"] == 12
+    # the partial last round: 384 workgroups on 256 CUs split their last 128; on 128 CUs they are three whole rounds
+    assert ops.attn_plan(4, 24, 24, 1024, 128, 8192, compute_units=128)["n_splits"] == 1
 
 
 def test_no_cpu_fallback():
@@ -222,8 +285,8 @@ def test_one_call_entry_point_validates_both_halves():
 
 
 def test_stream_probe_validates_before_launching():
-    """The tile-stream measurement aid refuses bad arguments with a status code (no GPU needed)."""
-    lib = _capi.lib()
+    """The tile-stream probe of the measurement library refuses bad arguments with a status code (no GPU needed)."""
+    lib = _capi.probe_lib()
     fake = ctypes.c_void_p(4096)
     region = 23 * 16384
     assert lib.we_stream_probe(None, 96 * region, 192, 23, 2, None) == -1            # null buffer
@@ -384,7 +447,7 @@ int main(void) {
     lib = _capi.lib()
     assert int(version) == lib.we_version()
     assert int(rc_null) == -1                                    # WE_ERR_NULL_POINTER
-    assert int(ws) == 4 * 16 * 256 * (128 * 2 + 16)
+    assert int(ws) == _capi.WE_WS_COUNTER_BYTES + 4 * 16 * 256 * (128 * 2 + 16)
     assert "workspace" in msg
 
 

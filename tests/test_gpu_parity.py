@@ -9,9 +9,9 @@ import pytest
 import torch
 
 from oracle import ring_oracle as ro
-from _harness import Pair, assert_attn_close, assert_bits_equal, merged_views, to_dev, MAX_ABS, MEAN_ABS
+from _harness import Pair, assert_attn_close, assert_bits_equal, assert_margin, merged_views, to_dev, MAX_ABS, MEAN_ABS
 import world_engine_amd as wea
-from world_engine_amd import ops
+from world_engine_amd import _capi, ops
 
 pytestmark = pytest.mark.gpu
 
@@ -149,7 +149,7 @@ def test_attention_cfg1_all_32_steps(gpu_device):
     """Benchmark configuration 1: B=1,H=16,Dh=128,T=256, 16 slots, 32 steps (warm-up + steady wrap)."""
     p = Pair(gpu_device, torch.bfloat16, B=1, H=16, Hkv=16, T=256, Dh=128, n_slots=16, cfg_id=1)
     worst = _run_and_check(p, 32)
-    _say(f"cfg1: worst max-abs {worst[0]:.2e} mean-abs {worst[1]:.2e}")
+    assert_margin("cfg1", worst)
 
 
 @pytest.mark.parametrize("n_splits", [1, 2, 3, 7, 16])
@@ -239,7 +239,7 @@ def test_attention_partial_round_tail_split(gpu_device):
     assert ops.attn_auto_splits(1, 160, 160, 256, 64, 512) == 1
     assert ops.attn_workspace_bytes(1, 160, 160, 256, 64, 512) == 0
     assert ops.attn_auto_splits(1, 320, 320, 256, 64, 512) == 2
-    assert ops.attn_workspace_bytes(1, 320, 320, 256, 64, 512) == 2 * 64 * 256 * (64 * 2 + 16)
+    assert ops.attn_workspace_bytes(1, 320, 320, 256, 64, 512) == _capi.WE_WS_COUNTER_BYTES + 2 * 64 * 256 * (64 * 2 + 16)
     p = Pair(gpu_device, torch.bfloat16, B=1, H=320, Hkv=320, T=256, Dh=64, n_slots=2, cfg_id=27)
     _run_and_check(p, 4)
     p = Pair(gpu_device, torch.bfloat16, B=1, H=160, Hkv=160, T=256, Dh=64, n_slots=2, cfg_id=27)
@@ -287,7 +287,7 @@ def test_attention_cfg2_full_depth_24_layers(gpu_device):
                 worst = (max(worst[0], mx), max(worst[1], mean))
         for layer in range(L_):
             p.assert_state_equal(layer=layer, what=f"t={t} layer={layer}")
-    _say(f"cfg2 full depth: worst max-abs {worst[0]:.2e} mean-abs {worst[1]:.2e}")
+    assert_margin("cfg2", worst)
 
 
 def test_attention_cfg4_frozen_substeps_schedule(gpu_device):
@@ -295,14 +295,14 @@ def test_attention_cfg4_frozen_substeps_schedule(gpu_device):
     call per frame.  State is compared after every call; outputs on the first frames and around
     the wrap."""
     p = Pair(gpu_device, torch.bfloat16, B=1, H=16, Hkv=16, T=256, Dh=128, n_slots=32, cfg_id=4)
-    _run_and_check(p, 35, frozen_subs=4, check_steps={0, 1, 31, 32, 34})
+    assert_margin("cfg4", _run_and_check(p, 35, frozen_subs=4, check_steps={0, 1, 31, 32, 34}))
 
 
 def test_attention_cfg3_full_size(gpu_device):
     """Benchmark configuration 3 at full size (B=4,H=24,T=1024, 8 slots): oracle on three steps, plus
     size-independent properties on the steady state."""
     p = Pair(gpu_device, torch.bfloat16, B=4, H=24, Hkv=24, T=1024, Dh=128, n_slots=8, cfg_id=3)
-    _run_and_check(p, 10, check_steps={0, 9})
+    assert_margin("cfg3", _run_and_check(p, 10, check_steps={0, 9}))
     # steady state: permuting the visible slots' contents must not change the result
     q, k, v, pos = p.inputs(10)
     p.set_frozen(True)
@@ -522,7 +522,7 @@ def test_hip_graph_replay_matches_eager(gpu_device):
     layer = p.hip.layers[0]
     out_s = torch.empty(1, 4, 128, 128, dtype=torch.bfloat16, device=dev)
     n_splits = 2
-    ws = torch.empty(ops.attn_workspace_bytes(1, 4, 4, 128, 128, layer.L, n_splits), dtype=torch.uint8, device=dev)
+    ws = ops.new_workspace(ops.attn_workspace_bytes(1, 4, 4, 128, 128, layer.L, n_splits), dev)
 
     def step():
         q_rot = ops.rope_kv_store(qs, ks, vs, pos_s, p.rope.cos, p.rope.sin, p.Hgrid, p.W, layer.kv,

@@ -21,11 +21,14 @@ def _both(p, t, n_splits=0, q_tile=0):
     (q_o, k_all, v_all, mask), (q_h, ring) = p.store(q, k, v, pos)
     base = ops.attn_ring(q_h, ring.kv, ring.written, ring.t_pos, ring.L, ring.dilation, n_splits=n_splits, q_tile=q_tile)
     out = torch.full_like(base, float("nan"))
+    torch.cuda.synchronize()
     before = torch.cuda.memory_allocated()
+    free_before = torch.cuda.mem_get_info()[0]        # hipMemGetInfo: what the driver itself has handed out
     ops.attn_ring_static(q_h, ring.kv, ring.written, ring.t_pos, ring.L, ring.dilation, out, n_splits=n_splits,
                          q_tile=q_tile)
-    assert torch.cuda.memory_allocated() == before, "the static entry point must not allocate through torch"
     torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before, "the static entry point must not allocate through torch"
+    assert torch.cuda.mem_get_info()[0] == free_before, "the static entry point must not allocate device memory at all"
     return out, base, ro.attention_fp32(q_o, k_all, v_all, mask)
 
 
@@ -71,3 +74,41 @@ def test_static_scratch_limit_and_unsplit_calls(gpu_device):
     # argument errors are those of we_attn_ring_fwd
     assert lib.we_attn_ring_fwd_static(None, s3, fake, fake, fake, fake, s3, 1, 1, 1, 64, 64, 64, 1, 0.1, 1, 0, 0, None) == -1
     assert lib.we_attn_ring_fwd_static(fake, s3, fake, fake, fake, fake, s3, 1, 1, 1, 64, 96, 64, 1, 0.1, 1, 0, 0, None) == -3
+
+
+def test_static_entry_point_under_graph_capture(gpu_device):
+    """What the entry point is for: captured into a HIP graph (after the device's one-time set-up,
+    which an eager call or ops.init() does and a capture cannot), replayed with eager work and
+    synchronisations in between, every replay compared with the workspace entry point's result."""
+    dev = gpu_device
+    ops.init(dev)
+    p = Pair(dev, torch.bfloat16, B=1, H=8, Hkv=8, T=128, Dh=128, n_slots=4, cfg_id=74)
+    eager = Pair(dev, torch.bfloat16, B=1, H=8, Hkv=8, T=128, Dh=128, n_slots=4, cfg_id=74)
+    p.set_frozen(False)
+    eager.set_frozen(False)
+    layer = p.hip.layers[0]
+    q_s = torch.empty(1, 8, 128, 128, dtype=torch.bfloat16, device=dev)
+    out_s = torch.empty(1, 8, 128, 128, dtype=torch.bfloat16, device=dev)
+    t_s = torch.zeros(1, 128, dtype=torch.long, device=dev)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                    # one eager call before the capture
+        ops.attn_ring_static(q_s, layer.kv, layer.written, t_s, layer.L, 1, out_s, n_splits=3)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ops.attn_ring_static(q_s, layer.kv, layer.written, t_s, layer.L, 1, out_s, n_splits=3)
+    for t in range(6):
+        q, k, v, pos = p.inputs(t)
+        (q_o, k_all, v_all, mask), (q_h, ring) = p.store(q, k, v, pos, strided=False)     # eager store into the captured cache
+        q_s.copy_(q_h)
+        t_s.fill_(t)
+        graph.replay()
+        torch.cuda.synchronize()
+        (_, _, _, _), (q_e, ring_e) = eager.store(q, k, v, pos, strided=False)
+        base = eager.attend(q_e, ring_e, n_splits=3, token_major_out=False)
+        assert torch.equal(out_s, base), f"replay {t}: static entry point under a graph differs from the workspace entry point"
+        assert_attn_close(out_s, ro.attention_fp32(q_o, k_all, v_all, mask), f"replay {t}")
+    assert torch.cuda.mem_get_info()[0] >= free_before - (8 << 20), "replays must not grow device memory"

@@ -1,7 +1,9 @@
-"""ctypes binding of the C ABI declared in ``include/we_attn.h``.
+"""ctypes binding of the C ABI declared in ``include/we_attn.h`` (``libwe_attn.so``, the product)
+and of the measurement library declared in ``include/we_attn_probe.h`` (``libwe_probe.so``, loaded
+only by the benchmark and by the tests of its entry points).
 
-The shared library is built in-tree by ``world_engine_amd/build.py`` (``hipcc`` for gfx950).
-There is no fallback: if the library is missing, every call raises.
+Both are built in-tree by ``world_engine_amd/build.py`` (``hipcc`` for gfx950).  There is no
+fallback: if a library is missing, every call into it raises.
 """
 from __future__ import annotations
 
@@ -11,11 +13,16 @@ from ctypes import c_char_p, c_float, c_int32, c_int64, c_size_t, c_void_p, POIN
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libwe_attn.so")
+PROBE_LIB_PATH = os.path.join(_HERE, "libwe_probe.so")
 
 WE_DTYPE_BF16, WE_DTYPE_F16, WE_DTYPE_F32 = 0, 1, 2
 WE_MAX_SLOTS = 256
 WE_STATIC_SCRATCH_BYTES = 32 << 20
+WE_WS_COUNTER_BYTES = 16384
+WE_SPLIT_TWO_PASS = 0x10000
+WE_PLAN_FIELDS = 6
 WE_ERR_SCRATCH_LIMIT = -7
+WE_ERR_NOT_READY = -8
 
 _I64x3 = POINTER(c_int64)
 
@@ -55,7 +62,10 @@ SIGNATURES = {
         c_int32, c_int32, c_int32, c_int32,        # B H T Dh
         c_int32, c_void_p,                         # dtype, stream
     ]),
+    "we_init": (c_int32, []),
     "we_attn_auto_splits": (c_int32, [c_int32, c_int32, c_int32, c_int32, c_int32, c_int64]),
+    "we_attn_plan": (c_int32, [c_int32, c_int32, c_int32, c_int32, c_int32, c_int64, c_int32, c_int32, c_int32, c_int32,
+                               POINTER(c_int32)]),
     "we_attn_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32, c_int32, c_int64, c_int32, c_int32]),
     "we_attn_ring_fwd": (c_int32, [
         c_void_p, _I64x3,                          # q, q_strides
@@ -65,16 +75,6 @@ SIGNATURES = {
         c_int32, c_int32, c_int32, c_int32, c_int32, c_int64,   # B H Hkv T Dh L
         c_int32, c_float, c_int32, c_int32, c_int32, c_void_p,  # dilation scale n_splits q_tile dtype stream
     ]),
-    "we_attn_ring_fwd_clocked": (c_int32, [
-        c_void_p, _I64x3,                          # q, q_strides
-        c_void_p, c_void_p, c_void_p,              # kv, written, t_pos
-        c_void_p, _I64x3,                          # out, out_strides
-        c_void_p, c_size_t,                        # workspace, bytes
-        c_int32, c_int32, c_int32, c_int32, c_int32, c_int64,   # B H Hkv T Dh L
-        c_int32, c_float, c_int32, c_int32, c_int32,            # dilation scale n_splits q_tile dtype
-        c_void_p, c_size_t, c_void_p,              # clocks, clocks_len, stream
-    ]),
-    "we_stream_probe": (c_int32, [c_void_p, c_size_t, c_int32, c_int32, c_int32, c_void_p]),
     "we_attn_ring_fwd_static": (c_int32, [
         c_void_p, _I64x3,                          # q, q_strides
         c_void_p, c_void_p, c_void_p,              # kv, written, t_pos
@@ -120,6 +120,21 @@ SIGNATURES = {
     ]),
 }
 
+# the measurement library exports these on top of everything above; must list every symbol
+# include/we_attn_probe.h declares
+PROBE_SIGNATURES = {
+    "we_attn_ring_fwd_clocked": (c_int32, [
+        c_void_p, _I64x3,                          # q, q_strides
+        c_void_p, c_void_p, c_void_p,              # kv, written, t_pos
+        c_void_p, _I64x3,                          # out, out_strides
+        c_void_p, c_size_t,                        # workspace, bytes
+        c_int32, c_int32, c_int32, c_int32, c_int32, c_int64,   # B H Hkv T Dh L
+        c_int32, c_float, c_int32, c_int32, c_int32,            # dilation scale n_splits q_tile dtype
+        c_void_p, c_size_t, c_void_p,              # clocks, clocks_len, stream
+    ]),
+    "we_stream_probe": (c_int32, [c_void_p, c_size_t, c_int32, c_int32, c_int32, c_void_p]),
+}
+
 _lib = None
 
 
@@ -138,6 +153,24 @@ def lib() -> ctypes.CDLL:
             fn.restype, fn.argtypes = res, args
         _lib = handle
     return _lib
+
+
+_probe_lib = None
+
+
+def probe_lib() -> ctypes.CDLL:
+    """Load the measurement library once (benchmark and probe tests only); raise if it has not
+    been built.  It carries its own copy of the product's entry points and per-device state."""
+    global _probe_lib
+    if _probe_lib is None:
+        if not os.path.exists(PROBE_LIB_PATH):
+            raise RuntimeError(f"{PROBE_LIB_PATH} is missing (run `python -m world_engine_amd.build`)")
+        handle = ctypes.CDLL(PROBE_LIB_PATH)
+        for name, (res, args) in {**SIGNATURES, **PROBE_SIGNATURES}.items():
+            fn = getattr(handle, name)
+            fn.restype, fn.argtypes = res, args
+        _probe_lib = handle
+    return _probe_lib
 
 
 def check(code: int, what: str) -> None:

@@ -198,16 +198,30 @@ class RingAttn(nn.Module):
     def from_reference(cls, src: nn.Module, config, rope: RoPE, merged_qkv: bool = True,
                        fuse_elementwise: bool = False, fuse_projection: bool = False):
         """Build from an ``Attn``-like module (anything with ``layer_idx`` and a matching state
-        dict), the way the reference's ``MergedQKVAttn(src, config)`` does."""
+        dict), the way the reference's ``MergedQKVAttn(src, config)`` does
+        (``src/patch_model.py:92-114``): same device and dtype as the source's weights, its
+        train / eval mode, ``q_proj | k_proj | v_proj`` rows concatenated into ``qkv_proj`` (or
+        split again when ``merged_qkv`` is off and the source is already merged).  Where the
+        reference loads with ``strict=False``, a key that has no place in the new module - or a
+        parameter of the new module that the source does not provide - raises here: a silently
+        random projection is not a state anyone wants."""
         new = cls(config, src.layer_idx, rope, merged_qkv=merged_qkv, fuse_elementwise=fuse_elementwise,
                   fuse_projection=fuse_projection)
         ref_w = next(src.parameters())
         new.to(device=ref_w.device, dtype=ref_w.dtype)
-        state = {k: v for k, v in src.state_dict().items()}
+        state = {k: v for k, v in src.state_dict().items() if not k.startswith("rope.")}
         if merged_qkv and "q_proj.weight" in state:
             state["qkv_proj.weight"] = torch.cat(
                 [state.pop("q_proj.weight"), state.pop("k_proj.weight"), state.pop("v_proj.weight")], dim=0)
-        new.load_state_dict(state, strict=False)
+        elif not merged_qkv and "qkv_proj.weight" in state:
+            q_w, k_w, v_w = state.pop("qkv_proj.weight").split((new.q_out, new.kv_out, new.kv_out), dim=0)
+            state.update({"q_proj.weight": q_w, "k_proj.weight": k_w, "v_proj.weight": v_w})
+        own = {k for k in new.state_dict() if not k.startswith("rope.")}
+        missing, unexpected = sorted(own - set(state)), sorted(set(state) - own)
+        if missing or unexpected:
+            raise RuntimeError(f"cannot build RingAttn from {type(src).__name__} (layer {src.layer_idx}): "
+                               f"missing keys {missing}, unexpected keys {unexpected}")
+        new.load_state_dict(state, strict=False)      # (strict=False only for the shared rope's buffers)
         new.train(src.training)
         return new
 
@@ -282,15 +296,26 @@ class RingAttn(nn.Module):
         return self.out_proj(y), v1
 
 
-def install_ring_attention(model: nn.Module, rope: RoPE, attn_types: tuple, merged_qkv: bool = True,
+def install_ring_attention(model: nn.Module, rope: Optional[RoPE], attn_types: tuple, merged_qkv: bool = True,
                            fuse_elementwise: bool = False, fuse_projection: bool = False) -> int:
     """Swap every submodule that is an instance of ``attn_types`` for a :class:`RingAttn`, the
     same ``set_submodule`` walk the reference uses for its merged-QKV patch
-    (``src/patch_model.py:144-147``).  Returns the number of modules replaced."""
+    (``src/patch_model.py:144-147``).  ``rope=None`` takes the tables of the modules' own ``.rope``
+    (``cos`` / ``sin`` buffers, grid from ``model.config.height / width``): modules that share one
+    rotary module (``src/model/world_model.py:199-202``) share one :class:`RoPE` afterwards too.
+    Returns the number of modules replaced."""
     n = 0
+    ropes = {}
     for name, mod in list(model.named_modules()):
         if isinstance(mod, attn_types) and not isinstance(mod, RingAttn):
-            model.set_submodule(name, RingAttn.from_reference(mod, model.config, rope, merged_qkv, fuse_elementwise,
+            r = rope
+            if r is None:
+                src = mod.rope
+                if id(src) not in ropes:
+                    ropes[id(src)] = RoPE(src.cos.detach().clone(), src.sin.detach().clone(), model.config.height,
+                                          model.config.width).to(src.cos.device)
+                r = ropes[id(src)]
+            model.set_submodule(name, RingAttn.from_reference(mod, model.config, r, merged_qkv, fuse_elementwise,
                                                                  fuse_projection))
             n += 1
     return n

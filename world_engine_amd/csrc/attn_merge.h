@@ -1,0 +1,105 @@
+// Merge of split-context partial results (gfx950): one output item = 8 consecutive head-dim
+// columns of one query row.  The same function serves the second-pass kernel (attn_combine.hip)
+// and the main kernel's own merge by the last workgroup to arrive (attn_ring.hip), so that both
+// routes produce identical bits.
+#pragma once
+#include "attn_mma.h"
+#include "we_kernels.h"
+
+namespace we {
+
+// 16-byte load of partial results.  L2: the load must not be served from this CU's vector L1
+// (the partials were written by other CUs of the same XCD a moment ago and live in its L2).
+template <bool L2>
+__device__ __forceinline__ u32x4_t load_partial16(const void* base, int64_t byte_off) {
+  if (L2) {
+    const __amdgpu_buffer_rsrc_t rs =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)0xffffffffu, 0x00020000);
+    // (the host keeps the workspace of a call that merges this way below 4 GiB)
+    return __builtin_amdgcn_raw_buffer_load_b128(rs, (int)(uint32_t)byte_off, 0, 16 /* sc1: miss the vector L1 */);
+  }
+  return *reinterpret_cast<const u32x4_t*>(static_cast<const unsigned char*>(base) + byte_off);
+}
+
+// Every split left, per query row, its normalised output as fp16 values times a row scale r_s, its
+// reference m_s (log2 domain) and its sum l_s; the result is sum_s w_s r_s O_s / sum_s w_s with
+// w_s = 2^(m_s - max m) * l_s.  Splits are merged eight at a time with all sixteen loads of a batch
+// issued before the first use (a plain loop over a run-time split count would serialise one memory
+// round trip per split).
+struct PartialBatch {
+  f32x4_t ml[8];   // (m, l, row scale, -)
+  f16x8_t ov[8];
+};
+
+// Requests splits [s0, s0 + 8) of workspace row `wrow` (query row - ws_row0; `rows` = the
+// workspace's row count), columns [8 dg, 8 dg + 8).
+template <int DH, bool L2>
+__device__ __forceinline__ void load_batch(PartialBatch& pb, const AttnParams& p, int64_t rows, int64_t wrow, int dg, int s0) {
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    if (s0 + j < p.n_splits) {  // (uniform: a request is 16 cycles of the CU's address path whether wanted or not)
+      const int64_t r = (int64_t)(s0 + j) * rows + wrow;
+      pb.ml[j] = __builtin_bit_cast(f32x4_t, load_partial16<L2>(p.ws_ml, r * 16));
+      pb.ov[j] = __builtin_bit_cast(f16x8_t, load_partial16<L2>(p.ws_o, (r * DH + dg * 8) * 2));
+    } else {
+      pb.ml[j] = f32x4_t{-INFINITY, 0.f, 0.f, 0.f};
+      pb.ov[j] = f16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+  }
+}
+
+// Adds the batch's first `n_valid` splits to the running (reference, denominator, numerators).
+__device__ __forceinline__ void accumulate_batch(const PartialBatch& pb, int n_valid, float& mmax, float& den, float (&acc)[8]) {
+  float bmax = mmax;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) bmax = fmaxf(bmax, pb.ml[j][0]);
+  const float carry = bmax > -INFINITY ? __builtin_amdgcn_exp2f(mmax - bmax) : 0.f;  // 0 on the first batch
+  den *= carry;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) acc[j] *= carry;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    // a part past the end, or one without keys, contributes nothing - not even 0 * inf
+    if (j < n_valid && pb.ml[j][1] > 0.f) {
+      const float w = __builtin_amdgcn_exp2f(pb.ml[j][0] - bmax) * pb.ml[j][1];
+      den += w;
+      const float wr = w * pb.ml[j][2];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += wr * (float)pb.ov[j][e];
+    }
+  }
+  mmax = bmax;
+}
+
+// Normalises, applies the head gate and stores columns [8 dg, 8 dg + 8) of query row (b, h, t).
+template <typename M>
+__device__ __forceinline__ void finish_item(const AttnParams& p, const float (&acc)[8], float den, int b, int h, int t, int dg) {
+  typedef typename M::frag_t frag_t;
+  const float inv = 1.f / den;
+  uint16_t* dst = reinterpret_cast<uint16_t*>(p.out) + b * p.os_b + h * p.os_h + (int64_t)t * p.os_t + dg * 8;
+  frag_t y = M::pack8(acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv, acc[4] * inv, acc[5] * inv,
+                      acc[6] * inv, acc[7] * inv);
+  if (p.gate != nullptr || p.gate_w != nullptr) {  // y * gate on element-type values, as the module's own multiply
+    const float g = head_gate<typename M::elem_t>(p, b, h, t);
+    y = M::pack8((float)y[0] * g, (float)y[1] * g, (float)y[2] * g, (float)y[3] * g, (float)y[4] * g,
+                 (float)y[5] * g, (float)y[6] * g, (float)y[7] * g);
+  }
+  *reinterpret_cast<frag_t*>(dst) = y;
+}
+
+// One output item, any number of splits.
+template <typename M, int DH, bool L2>
+__device__ __forceinline__ void merge_item(const AttnParams& p, int64_t rows, int64_t wrow, int b, int h, int t, int dg) {
+  float mmax = -INFINITY, den = 0.f;
+  float acc[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+  for (int s0 = 0; s0 < p.n_splits; s0 += 8) {
+    PartialBatch pb;
+    load_batch<DH, L2>(pb, p, rows, wrow, dg, s0);
+    accumulate_batch(pb, p.n_splits - s0, mmax, den, acc);
+  }
+  finish_item<M>(p, acc, den, b, h, t, dg);
+}
+
+}  // namespace we

@@ -31,8 +31,11 @@
 // run on the matrix cores while the VALU handles block i); LDS fragment reads are stated up to 15
 // reads ahead of their MFMAs, also across steps and barriers, and the order is pinned with
 // sched_barrier.  When the workgroup count leaves a partial last round of CUs, only that round's
-// (batch, kv head) units are context-split (see the planner in capi.hip); split workgroups leave
-// normalised partial outputs that attn_combine.hip merges.
+// (batch, kv head) units are context-split (see the planner in attn_plan.h); split workgroups leave
+// normalised partial outputs.  Those are merged either by a second kernel (attn_combine.hip), or -
+// when the planner could place all workgroups of a unit on one XCD - by this kernel itself: the
+// parts of a query tile count their arrivals and whichever finishes last merges them, reading the
+// others' rows out of the XCD's L2 (no second launch, no trip of the partials through HBM).
 //
 // The grid is 3-D (8 * query tiles, query heads per kv head, rounds of 8 units): no division by
 // run-time values is needed to find a workgroup's unit, and blockIdx.x % 8 is the XCD it runs on,
@@ -43,11 +46,10 @@
 // of a slot is loaded with its missing rows clamped and its missing keys masked to -inf.
 //
 // Roofline: 4*T*N_vis*Dh flops and 4*N_vis*Dh bytes of K/V per (batch, kv head).
-#include "attn_mma.h"
-#include "we_kernels.h"
-#include "../../include/we_attn.h"
+#include "attn_merge.h"
+#include "attn_plan.h"
+#include "device_state.h"
 
-#include <atomic>
 #include <type_traits>
 
 namespace we {
@@ -96,7 +98,8 @@ __device__ __forceinline__ u32x2_t lds_read_tr(const unsigned char* smem, uint32
 
 // RAGGED: the frame length is not a multiple of the 64-key tile (separate instantiation: the
 // masking of the short tiles costs registers the common case cannot spare).
-template <typename M, int DH, int KSPLIT, bool RAGGED>
+// CLOCKED: measurement library only - every workgroup reports its duration (p.clock_out).
+template <typename M, int DH, int KSPLIT, bool RAGGED, bool CLOCKED>
 __global__ void __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_per_eu(2, 2)))
 attn_ring_kernel(AttnParams p) {
   typedef typename M::frag_t frag_t;
@@ -118,9 +121,9 @@ attn_ring_kernel(AttnParams p) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, hh = lane >> 5;
-  // measurement aid: shader-clock and constant-rate (100 MHz) counters at the workgroup's start
-  const uint64_t clk0 = p.clock_out != nullptr ? (uint64_t)__builtin_readcyclecounter() : 0;
-  const uint64_t wall0 = p.clock_out != nullptr ? (uint64_t)__builtin_amdgcn_s_memrealtime() : 0;
+  // shader-clock and constant-rate (100 MHz) counters at the workgroup's start
+  const uint64_t clk0 = CLOCKED ? (uint64_t)__builtin_readcyclecounter() : 0;
+  const uint64_t wall0 = CLOCKED ? (uint64_t)__builtin_amdgcn_s_memrealtime() : 0;
   const int qb = wave % QW;   // query block of this wavefront
   const int hb = wave / QW;   // key block of every tile it handles when KSPLIT == 2 (else 0)
 
@@ -133,17 +136,30 @@ attn_ring_kernel(AttnParams p) {
   // to XCDs round-robin in linear order, so XCD = blockIdx.x % 8, and the workgroups that share
   // one K/V stream (the x * y of one round) all land on the same XCD and its L2.
   const int xcd = blockIdx.x & 7, qtile = blockIdx.x >> 3, hq_in = blockIdx.y;
-  const int us_raw = blockIdx.z * 8 + xcd;
-  // a workgroup past the end computes the addresses of the last one and leaves further down, so
-  // that the requests above and below do not wait behind a branch
-  const int us = us_raw < p.unit_splits ? us_raw : p.unit_splits - 1;
   // leading units run unsplit; the rest are cut into n_splits context parts each
-  int unit, split, nsp;
-  if (us < p.units_whole) {
-    unit = us; split = 0; nsp = 1;
+  int unit, split, nsp, us_raw;
+  if (p.merge) {
+    // all parts of a unit on this XCD (the planner made both unit counts multiples of 8): rounds
+    // [0, units_whole / 8) hold the whole units, then every eight split units take n_splits rounds
+    const int zw = p.units_whole >> 3;
+    us_raw = 0;  // (the grid has no workgroup past the end)
+    if ((int)blockIdx.z < zw) {
+      unit = blockIdx.z * 8 + xcd; split = 0; nsp = 1;
+    } else {
+      const int zz = blockIdx.z - zw;
+      unit = p.units_whole + (zz / p.n_splits) * 8 + xcd; split = zz % p.n_splits; nsp = p.n_splits;
+    }
   } else {
-    const int r = us - p.units_whole;
-    unit = p.units_whole + r / p.n_splits; split = r % p.n_splits; nsp = p.n_splits;
+    us_raw = blockIdx.z * 8 + xcd;
+    // a workgroup past the end computes the addresses of the last one and leaves further down, so
+    // that the requests above and below do not wait behind a branch
+    const int us = us_raw < p.unit_splits ? us_raw : p.unit_splits - 1;
+    if (us < p.units_whole) {
+      unit = us; split = 0; nsp = 1;
+    } else {
+      const int r = us - p.units_whole;
+      unit = p.units_whole + r / p.n_splits; split = r % p.n_splits; nsp = p.n_splits;
+    }
   }
   const int b = unit / p.Hkv, hkv = unit - b * p.Hkv;
   const int h = hkv * p.group + hq_in;
@@ -669,6 +685,8 @@ attn_ring_kernel(AttnParams p) {
   half_wave_pair(l_run, lo, up);
   float l_tot = lo + up;
   m_ref *= lmul;  // from raw logits to the log2 domain the merges work in
+  // this kernel merges the context parts itself: every wavefront stays to the end
+  const bool merging = p.merge != 0 && nsp > 1;
 
   if (KSPLIT == 2) {
     // ---- the two wavefronts of a query block merge their (m, l, O) through LDS ----
@@ -684,7 +702,8 @@ attn_ring_kernel(AttnParams p) {
       mb[(DB * 4) * 64] = f32x4_t{m_ref, l_tot, 0.f, 0.f};
     }
     __syncthreads();
-    if (hb == 1) return;
+    if (hb == 1 && !merging) return;
+    if (hb == 0) {
     const f32x4_t ml1 = mb[(DB * 4) * 64];
     // a wavefront whose sum is zero saw no key (or only keys that vanish against its reference):
     // its reference must not take part in the maximum
@@ -704,9 +723,11 @@ attn_ring_kernel(AttnParams p) {
       l_tot = a0 * l_tot + a1 * l1;
       m_ref = mm;
     }
+    }
   }
 
   // ---- epilogue ----
+  if (KSPLIT == 1 || hb == 0) {
   const int64_t rows = (int64_t)p.B * p.H * p.T - p.ws_row0;  // rows in the workspace
   const bool valid = qrow < p.T;
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
@@ -716,7 +737,9 @@ attn_ring_kernel(AttnParams p) {
   if (gated && nsp == 1 && qrow < p.T) gate_v = head_gate<typename M::elem_t>(p, b, h, qrow);
   // A split leaves its partial output as fp16 values in [-1, 1] plus one fp32 scale per row (the
   // row's largest normalised magnitude): 11 significant bits whatever the element type, for the
-  // bytes of a bf16 row, and no overflow whatever V holds.
+  // bytes of a bf16 row, and no overflow for any finite V.  A row that holds an infinity keeps the
+  // plain normalised values (scale 1), so that only the columns concerned turn non-finite, as in a
+  // single pass; a row whose largest magnitude is too small for its reciprocal is scaled by 2^100.
   float mul = inv;
   if (nsp > 1) {
     float amax = 0.f;
@@ -727,10 +750,18 @@ attn_ring_kernel(AttnParams p) {
     float alo, aup;
     half_wave_pair(amax, alo, aup);
     amax = fmaxf(alo, aup);
-    mul = amax > 0.f ? 1.f / amax : 0.f;
+    float row_scale;
+    if (amax < INFINITY) {
+      const float a = fmaxf(amax, 0x1p-100f);
+      mul = 1.f / a;
+      row_scale = a * inv;
+    } else {
+      mul = inv;
+      row_scale = 1.f;
+    }
     if (valid && hh == 0)
       *reinterpret_cast<f32x4_t*>(p.ws_ml + ((int64_t)split * rows + (row - p.ws_row0)) * 4) =
-          f32x4_t{l_tot > 0.f ? m_ref : -INFINITY, l_tot, amax * inv, 0.f};
+          f32x4_t{l_tot > 0.f ? m_ref : -INFINITY, l_tot, row_scale, 0.f};
   }
 #pragma unroll
   for (int db = 0; db < DB; ++db) {
@@ -764,36 +795,154 @@ attn_ring_kernel(AttnParams p) {
       }
     }
   }
-  if (p.clock_out != nullptr && tid == 0) {
+  }  // (epilogue of the wavefronts that hold results)
+
+  // ---- merge of the context parts, shared out among the workgroups that computed them ----
+  // Every part has left its rows in the workspace with plain stores, i.e. in the L2 of the XCD that
+  // all parts of a unit run on.  Once a workgroup's own rows are there (its wavefronts' store
+  // counters at zero, then the barrier) it counts itself in on the tile's arrival word.  The merge
+  // of the tile's BM x Dh outputs is cut into one share per part: the workgroup that finds all
+  // others counted merges its own share at once; the others look at the word for a bounded time
+  // (the parts of a tile finish within a microsecond or two of each other) and merge their share
+  // when the count is complete, so that the merge costs every CU a share of the reads instead of
+  // one CU all of them.  A workgroup that will not wait (any longer) says so in the word and goes;
+  // the last to arrive takes the shares of those that left.  All of this goes through one word per
+  // tile, whose atomic operations are ordered, so every share is merged exactly once, after every
+  // part is in, and nobody waits without a limit.  Partial rows are read with loads that miss the
+  // CU's own L1; the arithmetic is the second-pass kernel's.  The word is zero again once every
+  // workgroup has stopped looking at it, which is how the next call expects to find it.
+  //   word: bits 7:0 parts arrived, 15:8 parts departed, 31:16 shares given up by their owners
+  if (merging) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    volatile uint32_t* todo = reinterpret_cast<volatile uint32_t*>(smem + L::MISC_OFF);
+    uint32_t* word = p.ws_ctr + xcd * host::kCtrPerXcd +
+                     ((((unit - p.units_whole) >> 3) * p.group + hq_in) * p.q_tiles + qtile);
+    const uint32_t parts = (uint32_t)nsp;
+    uint32_t departed = 0;
+    if (tid == 0) {
+      uint32_t mine = 0;
+      const uint32_t before = __hip_atomic_fetch_add(word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      if ((before & 0xffu) + 1u == parts) {
+        mine = (before >> 16) | (1u << split);  // last in: its own share and those given up
+      } else {
+        bool all_in = false;
+        if (p.merge_wait > 0) {
+          const uint64_t t0 = __builtin_amdgcn_s_memrealtime();  // constant 100 MHz counter
+          do {
+            __builtin_amdgcn_s_sleep(4);
+            all_in = (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & 0xffu) == parts;
+          } while (!all_in && __builtin_amdgcn_s_memrealtime() - t0 < (uint64_t)p.merge_wait);
+        }
+        if (!all_in) {
+          // giving up the share - unless everyone was in before the mark, in which case the last
+          // one in has not seen it and the share is still this workgroup's
+          const uint32_t seen = __hip_atomic_fetch_or(word, 1u << (16 + split), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+          all_in = (seen & 0xffu) == parts;
+        }
+        if (all_in) mine = 1u << split;
+      }
+      *todo = mine;
+      // This workgroup will not look at the word again: it departs now, so that the operation's
+      // round trip runs under the merge below.  The last to depart puts the word back to zero.
+      departed = __hip_atomic_fetch_add(word, 0x100u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    __syncthreads();
+    uint32_t shares = (uint32_t)__builtin_amdgcn_readfirstlane((int)*todo);
+    const int64_t rows = (int64_t)p.B * p.H * p.T - p.ws_row0;
+    const int64_t wrow0 = ((int64_t)b * p.H + h) * p.T - p.ws_row0 + qtile * BM;
+    const int t0 = qtile * BM;
+    constexpr int DG = DH / 8;
+    constexpr unsigned N = BM * DG;                       // (row, 8 columns) items of the tile
+    constexpr int MAXI = N / 2 / 512 > 0 ? N / 2 / 512 : 1;  // items per thread of the largest share (two parts)
+    for (; shares != 0u; shares &= shares - 1u) {
+      const unsigned k = (unsigned)__builtin_ctz(shares);
+      // 16 (Dh 128) or 8 consecutive lanes share a row: whole rows per request
+      const int lo = (int)(k * N / parts), hi = (int)((k + 1u) * N / parts);
+      if (p.n_splits <= 8) {
+        // one batch of loads per item; the next item's are requested before this item's arithmetic,
+        // so that a thread's items cost one trip to the L2 between them, not one each
+        PartialBatch cur, nxt;
+        int it = lo + tid;
+        bool ok = it < hi && t0 + it / DG < p.T;
+        if (ok) load_batch<DH, true>(cur, p, rows, wrow0 + it / DG, it % DG, 0);
+#pragma unroll
+        for (int i = 0; i < MAXI; ++i) {
+          const int itn = it + 512;
+          const bool okn = i + 1 < MAXI && itn < hi && t0 + itn / DG < p.T;
+          if (okn) load_batch<DH, true>(nxt, p, rows, wrow0 + itn / DG, itn % DG, 0);
+          if (ok) {
+            float mmax = -INFINITY, den = 0.f;
+            float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            accumulate_batch(cur, p.n_splits, mmax, den, acc);
+            finish_item<M>(p, acc, den, b, h, t0 + it / DG, it % DG);
+          }
+          cur = nxt;
+          it = itn;
+          ok = okn;
+        }
+      } else {
+        for (int it = lo + tid; it < hi; it += 512)
+          if (t0 + it / DG < p.T) merge_item<M, DH, true>(p, rows, wrow0 + it / DG, b, h, t0 + it / DG, it % DG);
+      }
+    }
+    if (tid == 0 && ((departed >> 8) & 0xffu) + 1u == parts)
+      __hip_atomic_store(word, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  }
+  if (CLOCKED && tid == 0) {
     const uint64_t wg = blockIdx.x + (uint64_t)gridDim.x * (blockIdx.y + (uint64_t)gridDim.y * blockIdx.z);
     p.clock_out[2 * wg] = (uint64_t)__builtin_readcyclecounter() - clk0;
     p.clock_out[2 * wg + 1] = (uint64_t)__builtin_amdgcn_s_memrealtime() - wall0;
   }
 }
 
-template <typename M, int DH, int KSPLIT, bool RAGGED>
-static hipError_t launch_ring_r(const AttnParams& p, hipStream_t stream) {
-  // the LDS limit of a kernel is a per-device setting: raise it once on every device that launches
-  // (a flag that two threads both find unset is set twice, which is harmless)
-  static std::atomic<bool> configured[64] = {};
-  const int lds = RingLds<DH>::kBytes;
-  int dev = 0;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return e;
-  if (dev < 0 || dev >= 64 || !configured[dev].load(std::memory_order_acquire)) {
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_ring_kernel<M, DH, KSPLIT, RAGGED>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    if (e != hipSuccess) return e;
-    if (dev >= 0 && dev < 64) configured[dev].store(true, std::memory_order_release);
-  }
+// WE_WITH_PROBES (the measurement library's build) adds the CLOCKED instantiations; the product's
+// objects hold none of their code.
+#ifdef WE_WITH_PROBES
+constexpr bool kWithProbes = true;
+#else
+constexpr bool kWithProbes = false;
+#endif
+
+template <typename M, int DH, int KSPLIT, bool RAGGED, bool CLOCKED>
+static hipError_t launch_ring_c(const AttnParams& p, hipStream_t stream) {
   const int rounds = (p.unit_splits + 7) / 8;
   const dim3 grid((unsigned)(8 * p.q_tiles), (unsigned)p.group, (unsigned)rounds);
-  hipLaunchKernelGGL((attn_ring_kernel<M, DH, KSPLIT, RAGGED>), grid, dim3(512), lds, stream, p);
+  hipLaunchKernelGGL((attn_ring_kernel<M, DH, KSPLIT, RAGGED, CLOCKED>), grid, dim3(512), RingLds<DH>::kBytes, stream, p);
   return hipGetLastError();
+}
+template <typename M, int DH, int KSPLIT, bool RAGGED>
+static hipError_t launch_ring_r(const AttnParams& p, hipStream_t stream) {
+  if constexpr (kWithProbes) {
+    if (p.clock_out != nullptr) return launch_ring_c<M, DH, KSPLIT, RAGGED, true>(p, stream);
+  }
+  return launch_ring_c<M, DH, KSPLIT, RAGGED, false>(p, stream);
 }
 template <typename M, int DH, int KSPLIT>
 static hipError_t launch_ring_t(const AttnParams& p, hipStream_t stream) {
   return p.T % BN == 0 ? launch_ring_r<M, DH, KSPLIT, false>(p, stream) : launch_ring_r<M, DH, KSPLIT, true>(p, stream);
+}
+
+// The kernels use more LDS than a launch may ask for by default; the limit is a per-device
+// setting of each kernel, raised once per device by the library's set-up (device_state.hip).
+template <typename M, int DH, int KSPLIT, bool RAGGED, bool CLOCKED>
+static hipError_t configure_one() {
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_ring_kernel<M, DH, KSPLIT, RAGGED, CLOCKED>),
+                             hipFuncAttributeMaxDynamicSharedMemorySize, RingLds<DH>::kBytes);
+}
+template <typename M, int DH>
+static hipError_t configure_family() {
+  hipError_t e = configure_one<M, DH, 1, false, false>();
+  if (e == hipSuccess) e = configure_one<M, DH, 1, true, false>();
+  if (e == hipSuccess) e = configure_one<M, DH, 2, false, false>();
+  if (e == hipSuccess) e = configure_one<M, DH, 2, true, false>();
+  if constexpr (kWithProbes) {
+    if (e == hipSuccess) e = configure_one<M, DH, 1, false, true>();
+    if (e == hipSuccess) e = configure_one<M, DH, 1, true, true>();
+    if (e == hipSuccess) e = configure_one<M, DH, 2, false, true>();
+    if (e == hipSuccess) e = configure_one<M, DH, 2, true, true>();
+  }
+  return e;
 }
 
 // The four (element type, head dim) families are compiled as separate objects (WE_RING_PART selects
@@ -802,21 +951,25 @@ static hipError_t launch_ring_t(const AttnParams& p, hipStream_t stream) {
 hipError_t launch_attn_ring_bf16_128(const AttnParams& p, int ksplit, hipStream_t stream) {
   return ksplit == 2 ? launch_ring_t<Bf16Mma, 128, 2>(p, stream) : launch_ring_t<Bf16Mma, 128, 1>(p, stream);
 }
+hipError_t configure_attn_ring_bf16_128() { return configure_family<Bf16Mma, 128>(); }
 #endif
 #if !defined(WE_RING_PART) || WE_RING_PART == 1
 hipError_t launch_attn_ring_bf16_64(const AttnParams& p, int ksplit, hipStream_t stream) {
   return ksplit == 2 ? launch_ring_t<Bf16Mma, 64, 2>(p, stream) : launch_ring_t<Bf16Mma, 64, 1>(p, stream);
 }
+hipError_t configure_attn_ring_bf16_64() { return configure_family<Bf16Mma, 64>(); }
 #endif
 #if !defined(WE_RING_PART) || WE_RING_PART == 2
 hipError_t launch_attn_ring_f16_128(const AttnParams& p, int ksplit, hipStream_t stream) {
   return ksplit == 2 ? launch_ring_t<F16Mma, 128, 2>(p, stream) : launch_ring_t<F16Mma, 128, 1>(p, stream);
 }
+hipError_t configure_attn_ring_f16_128() { return configure_family<F16Mma, 128>(); }
 #endif
 #if !defined(WE_RING_PART) || WE_RING_PART == 3
 hipError_t launch_attn_ring_f16_64(const AttnParams& p, int ksplit, hipStream_t stream) {
   return ksplit == 2 ? launch_ring_t<F16Mma, 64, 2>(p, stream) : launch_ring_t<F16Mma, 64, 1>(p, stream);
 }
+hipError_t configure_attn_ring_f16_64() { return configure_family<F16Mma, 64>(); }
 #endif
 
 }  // namespace we

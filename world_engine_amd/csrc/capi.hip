@@ -1,131 +1,44 @@
 // C ABI of the ring-buffer attention library: argument validation and kernel dispatch.
 // Declarations and the reference call sites each entry point replaces: include/we_attn.h.
 #include "../../include/we_attn.h"
+#include "attn_plan.h"
+#include "device_state.h"
 #include "we_kernels.h"
-
-#include <mutex>
-
-// Split-context partial results of we_attn_ring_fwd_static: part of the library's device image, so
-// that the entry point needs no allocation and no caller-owned workspace.  Every GPU the library
-// runs on holds its own copy at its own address; host code must never use the array's name as an
-// address (on the host it is a stand-in for the symbol), only what hipGetSymbolAddress returns
-// with the device in question current.
-static __device__ __align__(256) unsigned char scratch[WE_STATIC_SCRATCH_BYTES];
 
 namespace {
 
-// Device address of `scratch` on the current device, looked up once per device.
-int static_scratch(void** out) {
-  constexpr int kMaxDevices = 64;
-  static std::mutex mu;
-  static void* ptr[kMaxDevices] = {};
-  int dev = -1;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return WE_ERR_LAUNCH;
-  std::lock_guard<std::mutex> lock(mu);
-  if (ptr[dev] == nullptr) {
-    void* p = nullptr;
-    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) return WE_ERR_LAUNCH;
-    ptr[dev] = p;
-  }
-  *out = ptr[dev];
-  return WE_OK;
-}
+using we::host::aligned16;
+using we::host::AttnPlan;
+using we::host::DeviceState;
+using we::host::launch_attn;
+using we::host::plan_attn;
+using we::host::ring_shape_ok;
+using we::host::strides_ok;
+using we::host::variant_of;
+using we::host::workspace_bytes_of;
 
-bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
-
-int elem_bytes(int dtype) { return dtype == WE_DTYPE_F32 ? 4 : 2; }
-
-// element strides whose byte value keeps every row start 16-byte aligned
-bool strides_ok(const int64_t s[3], int dtype) {
-  const int per16 = 16 / elem_bytes(dtype);
-  return s[0] % per16 == 0 && s[1] % per16 == 0 && s[2] % per16 == 0;
-}
-
-int ring_shape_ok(int B, int H, int Hkv, int T, int Dh, int64_t L, int dilation) {
-  if (B <= 0 || H <= 0 || Hkv <= 0 || T <= 0 || Dh <= 0 || L <= 0 || dilation <= 0) return WE_ERR_BAD_SHAPE;
-  if (H % Hkv != 0 || L % T != 0 || (L / T) % dilation != 0) return WE_ERR_BAD_SHAPE;
-  return WE_OK;
-}
-
-struct AttnPlan {
-  int variant;      // 1: 128 queries per workgroup, 2: 256
-  int block_m;      // queries per workgroup
-  int n_splits;     // context splits of the units that are split (1: none)
-  int units_whole;  // leading (batch, kv head) units that are not split
-  int64_t ws_rows;  // query rows that go through the split-context workspace
+// The device a call will run on.  Without one (or while its set-up is impossible: first use under
+// stream capture) `rc` says why, and `state` is a stand-in so that argument errors are still
+// reported first.
+struct Dev {
+  int rc;
+  DeviceState state;
 };
-
-// Pick the kernel shape and the context splitting.
-//  * Shape: 256 queries per workgroup when that alone gives at least one workgroup per CU, else
-//    128 queries (two wavefronts share each query block and split every tile's keys).
-//  * Few workgroups (256-token frames): every unit is split into the same number of context
-//    parts - as many as fit the CUs in one round up to four parts, then as many as give 160 to
-//    240 workgroups (more for long contexts, fewer for many parts) - but never fewer than two
-//    64-key tiles per part.
-//  * Many workgroups that do not divide into whole rounds of 256 CUs (e.g. 384): only the units
-//    of the last, partial round are split, so that round finishes in a fraction of the time.
-AttnPlan plan_attn(int B, int H, int Hkv, int T, int64_t L, int n_splits, int variant) {
-  AttnPlan pl;
-  const int64_t wg256 = (int64_t)B * H * ((T + 255) / 256);
-  const int64_t wg128 = (int64_t)B * H * ((T + 127) / 128);
-  // 256 queries per workgroup when that alone fills the CUs - or when 128 would spill into a
-  // second round that 256 avoids (136 to 256 heads of a 256-token frame: one round of fat
-  // workgroups beats one and a bit rounds of thin ones by 5 to 17 %)
-  pl.variant = variant ? variant : ((T >= 256 && (wg256 >= 256 || wg128 > 256)) ? 2 : 1);
-  pl.block_m = pl.variant == 2 ? 256 : 128;
-  const int units = B * Hkv;
-  const int members = (H / Hkv) * ((T + pl.block_m - 1) / pl.block_m);
-  const int64_t wgs = (int64_t)units * members;
-  const int64_t tiles = L / 64;  // visible 64-key tiles at steady state
-  const int64_t max_s = tiles / 2 > 0 ? tiles / 2 : 1;
-  pl.units_whole = 0;
-  pl.n_splits = 1;
-  if (n_splits > 0) {
-    pl.n_splits = n_splits;
-  } else if (wgs < 256) {
-    // Never more workgroups than CUs (a second, nearly empty round costs a whole kernel's
-    // time); and when the context is cut four ways or more, fewer workgroups than CUs: a part's
-    // fixed costs do not shrink with its length, the partial results grow with the number of
-    // parts, and the board clocks the kernel lower the more CUs are busy (cfg1: 6 parts 25.1 us
-    // per frame-step, 8 parts 27.2; 24 rings: 653 against 717).  Measured over 8 to 160
-    // workgroups per call: the best count is about 240 workgroups for up to six parts and about
-    // 192 for more.
-    // Long contexts (32 slots of a 256-token frame and more) amortise the extra parts and the lower
-    // clock over longer loops: about 240 workgroups there too (cfg4: 7 parts 32.0 us per frame-step,
-    // 6 parts 32.8), and all 256 when that is exactly four parts (64 workgroups: 4 parts beat 3 by
-    // 2 to 7 %).
-    // Beyond sixteen parts every part's own cost weighs more: about 160 workgroups (4 heads: 20
-    // parts 21.2 to 27.2 us per frame-step over 16 to 64 slots, 24 parts 21.7 to 27.4).
-    int64_t s = 256 / wgs;
-    if (s > 4) s = ((wgs >= 40 || (tiles >= 96 && 240 / wgs <= 16)) ? 240 : (192 / wgs > 16 ? 160 : 192)) / wgs;
-    if (s > max_s) s = max_s;
-    if (s > 64) s = 64;
-    if (s < 1) s = 1;
-    pl.n_splits = (int)s;
-  } else if (wgs < 4 * 256 && members <= 256) {
-    const int whole_units = (int)((wgs / 256) * 256 / members);
-    const int64_t rem_wgs = (int64_t)(units - whole_units) * members;
-    if (rem_wgs > 0 && rem_wgs <= 128) {
-      int64_t s = 256 / rem_wgs;
-      if (s > 8) s = 8;
-      if (s > max_s / 2) s = max_s / 2;
-      if (s > 1) {
-        pl.n_splits = (int)s;
-        pl.units_whole = whole_units;
-      }
-    }
-  }
-  pl.ws_rows = pl.n_splits > 1 ? (int64_t)(units - pl.units_whole) * (H / Hkv) * T : 0;
-  return pl;
+Dev dev_for(hipStream_t st) {
+  const DeviceState* ds = nullptr;
+  Dev d;
+  d.rc = we::host::device_state(st, &ds);
+  d.state = ds ? *ds : DeviceState{256, false, nullptr};
+  return d;
 }
 
-int variant_of(int q_tile) {
-  switch (q_tile) {
-    case 0: return 0;
-    case 128: return 1;
-    case 256: return 2;
-    default: return -1;
-  }
+// prepare_attn for the device the call will run on
+int prepare_attn(const DeviceState& ds, const void* q, const int64_t* q_strides, const void* kv, const uint8_t* written,
+                 const int64_t* t_pos, void* out, const int64_t* out_strides, void* workspace, size_t workspace_bytes,
+                 int B, int H, int Hkv, int T, int Dh, int64_t L, int dilation, float scale, int n_splits, int q_tile,
+                 int dtype, we::AttnParams& p, AttnPlan& pl) {
+  return we::host::prepare_attn(q, q_strides, kv, written, t_pos, out, out_strides, workspace, workspace_bytes, B, H,
+                                Hkv, T, Dh, L, dilation, scale, n_splits, q_tile, dtype, ds.cus, ds.xcd_merge, p, pl);
 }
 
 // Validation of a we_rope_kv_store call and its kernel parameters.
@@ -166,62 +79,6 @@ int prepare_store(const void* q, const void* k, const void* v, const int64_t* q_
   p.B = B; p.H = H; p.Hkv = Hkv; p.T = T; p.Dh = Dh;
   p.dilation = dilation; p.num_buckets = (int)((L / T) / dilation); p.frozen = is_frozen ? 1 : 0;
   p.norm_eps = 0.f; p.v1 = nullptr; p.v_lamb = nullptr; p.v1s_b = p.v1s_h = p.v1s_t = 0;
-  return WE_OK;
-}
-
-// Validation of a we_attn_ring_fwd call, its plan and its kernel parameters.
-int prepare_attn(const void* q, const int64_t* q_strides, const void* kv, const uint8_t* written,
-                 const int64_t* t_pos, void* out, const int64_t* out_strides, void* workspace, size_t workspace_bytes,
-                 int B, int H, int Hkv, int T, int Dh, int64_t L, int dilation, float scale, int n_splits, int q_tile,
-                 int dtype, we::AttnParams& p, AttnPlan& pl) {
-  if (!q || !q_strides || !kv || !written || !t_pos || !out || !out_strides) return WE_ERR_NULL_POINTER;
-  int rc = ring_shape_ok(B, H, Hkv, T, Dh, L, dilation);
-  if (rc != WE_OK) return rc;
-  if (dtype != WE_DTYPE_BF16 && dtype != WE_DTYPE_F16 && dtype != WE_DTYPE_F32) return WE_ERR_UNSUPPORTED;
-  if (Dh != 64 && Dh != 128) return WE_ERR_UNSUPPORTED;
-  if (L / T > WE_MAX_SLOTS) return WE_ERR_UNSUPPORTED;
-  if ((uint64_t)(L + T) * (uint64_t)Dh * 2u >= (1ull << 32)) return WE_ERR_UNSUPPORTED;  // 32-bit tile offsets
-  if (!(scale > 0.f) || n_splits < 0 || n_splits > 64) return WE_ERR_BAD_SHAPE;
-  if (variant_of(q_tile) < 0) return WE_ERR_UNSUPPORTED;
-  if (dtype == WE_DTYPE_F32) {
-    // fp32 caches take the plain one-pass kernel: no context splitting, no tile choice
-    if (n_splits > 1 || H > 65535 || B > 65535) return WE_ERR_UNSUPPORTED;
-    n_splits = 1;
-  }
-  if (!aligned16(q) || !aligned16(kv) || !aligned16(out) || !strides_ok(q_strides, dtype) ||
-      !strides_ok(out_strides, dtype))
-    return WE_ERR_ALIGNMENT;
-
-  pl = plan_attn(B, H, Hkv, T, L, n_splits, variant_of(q_tile));
-  const size_t ws_need = (size_t)pl.n_splits * (size_t)pl.ws_rows * ((size_t)Dh * 2 + 4 * sizeof(float));
-  if (ws_need > 0) {
-    if (!workspace || !aligned16(workspace)) return WE_ERR_WORKSPACE;
-    if (workspace_bytes < ws_need) return WE_ERR_WORKSPACE;
-  }
-
-  p.q = q; p.kv = kv; p.written = written; p.t_pos = t_pos; p.out = out;
-  p.ws_o = ws_need ? static_cast<uint16_t*>(workspace) : nullptr;
-  p.ws_ml = ws_need ? reinterpret_cast<float*>(p.ws_o + (size_t)pl.n_splits * (size_t)pl.ws_rows * Dh) : nullptr;
-  p.qs_b = q_strides[0]; p.qs_h = q_strides[1]; p.qs_t = q_strides[2];
-  p.os_b = out_strides[0]; p.os_h = out_strides[1]; p.os_t = out_strides[2];
-  p.L = L;
-  p.B = B; p.H = H; p.Hkv = Hkv; p.T = T;
-  p.n_slots = (int)(L / T); p.dilation = dilation; p.num_buckets = p.n_slots / dilation;
-  p.n_splits = pl.n_splits;
-  p.units_whole = pl.units_whole;
-  p.ws_row0 = (int64_t)B * H * T - pl.ws_rows;
-  p.q_tiles = (T + pl.block_m - 1) / pl.block_m;
-  p.group = H / Hkv;
-  p.members = p.group * p.q_tiles;
-  p.unit_splits = pl.units_whole + (B * Hkv - pl.units_whole) * pl.n_splits;
-  p.scale_log2 = scale * 1.4426950408889634f;
-  p.gate = nullptr; p.gs_b = p.gs_h = p.gs_t = 0;
-  p.gate_x = nullptr; p.gate_w = nullptr; p.gx_b = p.gx_t = 0;
-  p.clock_out = nullptr;
-  p.q_dma = (q_strides[2] > 0 && (uint64_t)T * (uint64_t)q_strides[2] * 2u < (1ull << 31)) ? 1 : 0;
-
-  if ((p.unit_splits + 7) / 8 > 65535 || p.group > 65535 || (int64_t)B * H - (int64_t)pl.units_whole * p.group > 65535)
-    return WE_ERR_UNSUPPORTED;  // grid y / z limits of the two launches
   return WE_OK;
 }
 
@@ -299,17 +156,6 @@ int apply_gate_extras(const we_attn_extras* extras, int dtype, we::AttnParams& p
   return WE_OK;
 }
 
-int launch_attn(const we::AttnParams& p, const AttnPlan& pl, int Dh, int dtype, hipStream_t st) {
-  if (dtype == WE_DTYPE_F32) return we::launch_attn_ring_f32(p, Dh, st) == hipSuccess ? WE_OK : WE_ERR_LAUNCH;
-  const int ksplit = pl.variant == 1 ? 2 : 1;
-  hipError_t e;
-  if (dtype == WE_DTYPE_BF16) e = Dh == 128 ? we::launch_attn_ring_bf16_128(p, ksplit, st) : we::launch_attn_ring_bf16_64(p, ksplit, st);
-  else e = Dh == 128 ? we::launch_attn_ring_f16_128(p, ksplit, st) : we::launch_attn_ring_f16_64(p, ksplit, st);
-  if (e != hipSuccess) return WE_ERR_LAUNCH;
-  if (pl.n_splits > 1 && we::launch_attn_combine(p, Dh, dtype, st) != hipSuccess) return WE_ERR_LAUNCH;
-  return WE_OK;
-}
-
 }  // namespace
 
 extern "C" {
@@ -326,6 +172,7 @@ const char* we_error_string(int code) {
     case WE_ERR_WORKSPACE: return "split-context workspace missing or too small";
     case WE_ERR_LAUNCH: return "HIP runtime refused the kernel launch";
     case WE_ERR_SCRATCH_LIMIT: return "sizes need more split-context scratch than the library's static buffer (WE_STATIC_SCRATCH_BYTES) holds";
+    case WE_ERR_NOT_READY: return "first call on this device made under stream capture: call we_init() on the device beforehand";
     default: return "unknown error code";
   }
 }
@@ -375,19 +222,49 @@ int we_rope_apply(const void* x, const int64_t x_strides[3], void* x_out, const 
   return we::launch_rope_kv_store(p, dtype, static_cast<hipStream_t>(stream)) == hipSuccess ? WE_OK : WE_ERR_LAUNCH;
 }
 
+int we_init(void) { return we::host::init_current_device(); }
+
 int32_t we_attn_auto_splits(int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L) {
   (void)Dh;
   if (B <= 0 || H <= 0 || Hkv <= 0 || H % Hkv != 0 || T <= 0 || L <= 0) return 1;
-  return plan_attn(B, H, Hkv, T, L, 0, 0).n_splits;
+  return plan_attn(B, H, Hkv, T, L, 0, 0, we::host::compute_units(), false).n_splits;
 }
 
 size_t we_attn_workspace_bytes(int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L,
                                int32_t n_splits, int32_t q_tile) {
   if (B <= 0 || H <= 0 || Hkv <= 0 || H % Hkv != 0 || T <= 0 || Dh <= 0 || L <= 0 || n_splits < 0) return 0;
-  const int variant = variant_of(q_tile);
+  const int variant = variant_of(q_tile & ~WE_SPLIT_TWO_PASS);
   if (variant < 0) return 0;
-  const AttnPlan pl = plan_attn(B, H, Hkv, T, L, n_splits, variant);
-  return (size_t)pl.n_splits * (size_t)pl.ws_rows * ((size_t)Dh * 2 + 4 * sizeof(float));
+  return workspace_bytes_of(plan_attn(B, H, Hkv, T, L, n_splits, variant, we::host::compute_units(), false), Dh);
+}
+
+int we_attn_plan(int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L, int32_t n_splits,
+                 int32_t q_tile, int32_t compute_units, int32_t xcd_merge, int32_t plan[WE_PLAN_FIELDS]) {
+  if (!plan) return WE_ERR_NULL_POINTER;
+  if (B <= 0 || H <= 0 || Hkv <= 0 || H % Hkv != 0 || T <= 0 || Dh <= 0 || L <= 0 || L % T != 0 || n_splits < 0 ||
+      n_splits > 64 || compute_units < 0)
+    return WE_ERR_BAD_SHAPE;
+  const bool two_pass = (q_tile & WE_SPLIT_TWO_PASS) != 0;
+  const int variant = variant_of(q_tile & ~WE_SPLIT_TWO_PASS);
+  if (variant < 0) return WE_ERR_UNSUPPORTED;
+  const int cus = compute_units > 0 ? compute_units : we::host::compute_units();
+  if (xcd_merge < 0) {  // what the current device's set-up found
+    const DeviceState* ds = nullptr;
+    const int rc = we::host::device_state(nullptr, &ds);
+    if (rc != WE_OK) return rc;
+    xcd_merge = ds->xcd_merge ? 1 : 0;
+  }
+  AttnPlan pl = plan_attn(B, H, Hkv, T, L, n_splits, variant, cus, xcd_merge != 0 && !two_pass);
+  if (workspace_bytes_of(pl, Dh) >= (1ull << 32)) pl.merge = 0;
+  const int q_tiles = (T + pl.block_m - 1) / pl.block_m;
+  const int64_t wgs = (int64_t)q_tiles * (H / Hkv) * (pl.units_whole + (int64_t)(B * Hkv - pl.units_whole) * pl.n_splits);
+  plan[0] = pl.block_m;
+  plan[1] = pl.n_splits;
+  plan[2] = pl.units_whole;
+  plan[3] = pl.merge;
+  plan[4] = (int32_t)(wgs > 0x7fffffff ? 0x7fffffff : wgs);
+  plan[5] = cus;
+  return WE_OK;
 }
 
 int we_attn_ring_fwd(const void* q, const int64_t q_strides[3], const void* kv, const uint8_t* written,
@@ -395,44 +272,15 @@ int we_attn_ring_fwd(const void* q, const int64_t q_strides[3], const void* kv, 
                      size_t workspace_bytes, int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh,
                      int64_t L, int32_t dilation, float scale, int32_t n_splits, int32_t q_tile,
                      int32_t dtype, void* stream) {
-  we::AttnParams p;
-  AttnPlan pl;
-  const int rc = prepare_attn(q, q_strides, kv, written, t_pos, out, out_strides, workspace, workspace_bytes, B, H,
-                              Hkv, T, Dh, L, dilation, scale, n_splits, q_tile, dtype, p, pl);
-  if (rc != WE_OK) return rc;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  return launch_attn(p, pl, Dh, dtype, st);
-}
-
-int we_attn_ring_fwd_clocked(const void* q, const int64_t q_strides[3], const void* kv, const uint8_t* written,
-                             const int64_t* t_pos, void* out, const int64_t out_strides[3], void* workspace,
-                             size_t workspace_bytes, int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh,
-                             int64_t L, int32_t dilation, float scale, int32_t n_splits, int32_t q_tile,
-                             int32_t dtype, uint64_t* clocks, size_t clocks_len, void* stream) {
-  if (!clocks) return WE_ERR_NULL_POINTER;
-  if (dtype == WE_DTYPE_F32) return WE_ERR_UNSUPPORTED;
+  const Dev dev = dev_for(st);
   we::AttnParams p;
   AttnPlan pl;
-  const int rc = prepare_attn(q, q_strides, kv, written, t_pos, out, out_strides, workspace, workspace_bytes, B, H,
-                              Hkv, T, Dh, L, dilation, scale, n_splits, q_tile, dtype, p, pl);
+  const int rc = prepare_attn(dev.state, q, q_strides, kv, written, t_pos, out, out_strides, workspace,
+                              workspace_bytes, B, H, Hkv, T, Dh, L, dilation, scale, n_splits, q_tile, dtype, p, pl);
   if (rc != WE_OK) return rc;
-  const size_t wgs = (size_t)(8 * p.q_tiles) * (size_t)p.group * (size_t)((p.unit_splits + 7) / 8);
-  if (clocks_len < 2 * wgs) return WE_ERR_WORKSPACE;
-  p.clock_out = clocks;
-  return launch_attn(p, pl, Dh, dtype, static_cast<hipStream_t>(stream));
-}
-
-int we_stream_probe(const void* buf, size_t buf_bytes, int32_t workgroups, int32_t tiles, int32_t share, void* stream) {
-  if (!buf) return WE_ERR_NULL_POINTER;
-  if (workgroups <= 0 || workgroups % 8 != 0 || workgroups > 65536 || tiles <= 0 || tiles > 65536 || share <= 0 ||
-      (workgroups / 8) % share != 0)
-    return WE_ERR_BAD_SHAPE;
-  if (!aligned16(buf)) return WE_ERR_ALIGNMENT;
-  const uint64_t region = (uint64_t)tiles * 16384u;
-  if (region >= (1ull << 32)) return WE_ERR_UNSUPPORTED;  // 32-bit DMA offsets within a region
-  if ((uint64_t)(workgroups / share) * region > buf_bytes) return WE_ERR_WORKSPACE;
-  return we::launch_stream_probe(buf, workgroups, tiles, share, static_cast<hipStream_t>(stream)) == hipSuccess
-             ? WE_OK : WE_ERR_LAUNCH;
+  if (dev.rc != WE_OK) return dev.rc;
+  return launch_attn(p, pl, Dh, dtype, st);
 }
 
 int we_attn_ring_fwd_static(const void* q, const int64_t q_strides[3], const void* kv, const uint8_t* written,
@@ -440,22 +288,19 @@ int we_attn_ring_fwd_static(const void* q, const int64_t q_strides[3], const voi
                             int32_t Hkv, int32_t T, int32_t Dh, int64_t L, int32_t dilation, float scale,
                             int32_t n_splits, int32_t q_tile, int32_t dtype, void* stream) {
   // sizes first, so that a call that cannot fit is refused before anything else happens
-  if (B > 0 && H > 0 && Hkv > 0 && H % Hkv == 0 && T > 0 && Dh > 0 && L > 0 && n_splits >= 0 && variant_of(q_tile) >= 0 &&
-      dtype != WE_DTYPE_F32) {
-    const AttnPlan sz = plan_attn(B, H, Hkv, T, L, n_splits, variant_of(q_tile));
-    const unsigned long long need =
-        (unsigned long long)sz.n_splits * (unsigned long long)sz.ws_rows * ((unsigned long long)Dh * 2 + 4 * sizeof(float));
-    if (need > WE_STATIC_SCRATCH_BYTES) return WE_ERR_SCRATCH_LIMIT;
-  }
-  void* ws = nullptr;
-  int rc = static_scratch(&ws);
-  if (rc != WE_OK) return rc;
+  if (we_attn_workspace_bytes(B, H, Hkv, T, Dh, L, n_splits, q_tile) > WE_STATIC_SCRATCH_BYTES && dtype != WE_DTYPE_F32)
+    return WE_ERR_SCRATCH_LIMIT;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const Dev dev = dev_for(st);
+  // (a stand-in address keeps the argument checks of a call without a device those of we_attn_ring_fwd)
+  void* ws = dev.state.scratch ? dev.state.scratch : reinterpret_cast<void*>(uintptr_t{4096});
   we::AttnParams p;
   AttnPlan pl;
-  rc = prepare_attn(q, q_strides, kv, written, t_pos, out, out_strides, ws, WE_STATIC_SCRATCH_BYTES, B, H, Hkv, T, Dh,
-                    L, dilation, scale, n_splits, q_tile, dtype, p, pl);
+  const int rc = prepare_attn(dev.state, q, q_strides, kv, written, t_pos, out, out_strides, ws,
+                              WE_STATIC_SCRATCH_BYTES, B, H, Hkv, T, Dh, L, dilation, scale, n_splits, q_tile, dtype, p, pl);
   if (rc != WE_OK) return rc;
-  return launch_attn(p, pl, Dh, dtype, static_cast<hipStream_t>(stream));
+  if (dev.rc != WE_OK) return dev.rc;
+  return launch_attn(p, pl, Dh, dtype, st);
 }
 
 int we_rope_kv_attn_fwd(const void* q, const void* k, const void* v, const int64_t q_strides[3],
@@ -475,10 +320,12 @@ int we_rope_kv_attn_fwd(const void* q, const void* k, const void* v, const int64
   if (rc != WE_OK) return rc;
   // the attention reads the rotated q the store leaves in q_out, contiguous [B, H, T, Dh]
   const int64_t qo_strides[3] = {(int64_t)H * T * Dh, (int64_t)T * Dh, (int64_t)Dh};
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const Dev dev = dev_for(st);
   we::AttnParams p;
   AttnPlan pl;
-  rc = prepare_attn(q_out, qo_strides, kv, written, t_pos, out, out_strides, workspace, workspace_bytes, B, H, Hkv,
-                    T, Dh, L, dilation, scale, n_splits, q_tile, dtype, p, pl);
+  rc = prepare_attn(dev.state, q_out, qo_strides, kv, written, t_pos, out, out_strides, workspace, workspace_bytes, B,
+                    H, Hkv, T, Dh, L, dilation, scale, n_splits, q_tile, dtype, p, pl);
   if (rc != WE_OK) return rc;
   if (extras) {
     const we_attn_extras& x = *extras;
@@ -492,7 +339,7 @@ int we_rope_kv_attn_fwd(const void* q, const void* k, const void* v, const int64
     rc = apply_gate_extras(extras, dtype, p);
     if (rc != WE_OK) return rc;
   }
-  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dev.rc != WE_OK) return dev.rc;
   // Everything is validated before the first launch; the kernels follow each other on the stream.
   if (we::launch_rope_kv_store(sp, dtype, st) != hipSuccess) return WE_ERR_LAUNCH;
   return launch_attn(p, pl, Dh, dtype, st);
@@ -507,7 +354,10 @@ int we_qkv_rope_kv_store(const we_qkv_proj* proj, void* q_out, const float* cos_
   const int rc = prepare_proj(proj, q_out, cos_table, sin_table, table_rows, t_pos, y_pos, x_pos, pos_stride_b, grid_h,
                               grid_w, kv, written, B, H, Hkv, T, Dh, L, dilation, is_frozen, dtype, extras, pp);
   if (rc != WE_OK) return rc;
-  return we::launch_qkv_rope_store(pp, dtype, static_cast<hipStream_t>(stream)) == hipSuccess ? WE_OK : WE_ERR_LAUNCH;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const Dev dev = dev_for(st);  // (the kernel's LDS limit is raised by the device's set-up)
+  if (dev.rc != WE_OK) return dev.rc;
+  return we::launch_qkv_rope_store(pp, dtype, st) == hipSuccess ? WE_OK : WE_ERR_LAUNCH;
 }
 
 int we_qkv_rope_kv_attn_fwd(const we_qkv_proj* proj, void* q_out, const float* cos_table, const float* sin_table,
@@ -522,14 +372,16 @@ int we_qkv_rope_kv_attn_fwd(const we_qkv_proj* proj, void* q_out, const float* c
                         grid_w, kv, written, B, H, Hkv, T, Dh, L, dilation, is_frozen, dtype, extras, pp);
   if (rc != WE_OK) return rc;
   const int64_t qo_strides[3] = {(int64_t)H * T * Dh, (int64_t)T * Dh, (int64_t)Dh};
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const Dev dev = dev_for(st);
   we::AttnParams p;
   AttnPlan pl;
-  rc = prepare_attn(q_out, qo_strides, kv, written, t_pos, out, out_strides, workspace, workspace_bytes, B, H, Hkv,
-                    T, Dh, L, dilation, scale, n_splits, q_tile, dtype, p, pl);
+  rc = prepare_attn(dev.state, q_out, qo_strides, kv, written, t_pos, out, out_strides, workspace, workspace_bytes, B,
+                    H, Hkv, T, Dh, L, dilation, scale, n_splits, q_tile, dtype, p, pl);
   if (rc != WE_OK) return rc;
   rc = apply_gate_extras(extras, dtype, p);
   if (rc != WE_OK) return rc;
-  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dev.rc != WE_OK) return dev.rc;
   if (we::launch_qkv_rope_store(pp, dtype, st) != hipSuccess) return WE_ERR_LAUNCH;
   return launch_attn(p, pl, Dh, dtype, st);
 }

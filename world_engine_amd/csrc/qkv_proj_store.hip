@@ -24,9 +24,8 @@
 // Roofline: the weight matrix once (2 K N bytes) + x once; 2 T N K flops.
 #include "attn_mma.h"
 #include "rope_kv_store.h"
+#include "device_state.h"
 #include "we_kernels.h"
-
-#include <atomic>
 
 namespace we {
 
@@ -255,25 +254,26 @@ qkv_rope_store_kernel(ProjParams p) {
 
 template <typename M, typename Tag>
 static hipError_t launch_proj(const ProjParams& p, hipStream_t stream) {
-  static std::atomic<bool> configured[64];
-  int dev = 0;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return e;
-  auto kern = qkv_rope_store_kernel<M, Tag>;
-  if (dev < 0 || dev >= 64 || !configured[dev].load(std::memory_order_acquire)) {
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, PROJ_LDS_B);
-    if (e != hipSuccess) return e;
-    if (dev >= 0 && dev < 64) configured[dev].store(true, std::memory_order_release);
-  }
   const unsigned groups = (unsigned)((p.n_tiles + 7) / 8);
   const dim3 grid(8u * groups * (unsigned)(p.m_tiles * p.s.B));
-  hipLaunchKernelGGL(kern, grid, dim3(512), PROJ_LDS_B, stream, p);
+  hipLaunchKernelGGL((qkv_rope_store_kernel<M, Tag>), grid, dim3(512), PROJ_LDS_B, stream, p);
   return hipGetLastError();
 }
 
 hipError_t launch_qkv_rope_store(const ProjParams& p, int dtype, hipStream_t stream) {
   if (dtype == 0) return launch_proj<Bf16Mma, Bf16Tag>(p, stream);
   return launch_proj<F16Mma, F16Tag>(p, stream);
+}
+
+// The kernel's LDS ring exceeds the default per-launch limit: raised once per device by the
+// library's set-up (device_state.hip).
+hipError_t configure_qkv_rope_store() {
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&qkv_rope_store_kernel<Bf16Mma, Bf16Tag>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, PROJ_LDS_B);
+  if (e == hipSuccess)
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&qkv_rope_store_kernel<F16Mma, F16Tag>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, PROJ_LDS_B);
+  return e;
 }
 
 }  // namespace we

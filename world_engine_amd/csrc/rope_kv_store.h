@@ -82,7 +82,7 @@ __device__ __forceinline__ void rms_norm_chunk(Chunk16<Tag>& c, int cpr, int Dh,
   for (int i = 0; i < 16; ++i) c.e[i] = Tag::from_f32(x[i] * r);
 }
 
-// torch.lerp(v, v1, w) on 16 elements: fp32 arithmetic, the formula switches at w = 0.5
+// torch.lerp(v, v1, w) on 16 elements: fp32 arithmetic, the formula switches at |w| = 0.5
 // (ATen/native/Lerp.h), result rounded to the element type.
 template <typename Tag>
 __device__ __forceinline__ void lerp_chunk(Chunk16<Tag>& v, const Chunk16<Tag>& v1, float w) {
@@ -90,7 +90,7 @@ __device__ __forceinline__ void lerp_chunk(Chunk16<Tag>& v, const Chunk16<Tag>& 
   for (int i = 0; i < 16; ++i) {
     const float a = Tag::to_f32(v.e[i]), b = Tag::to_f32(v1.e[i]);
     const float d = b - a;
-    v.e[i] = Tag::from_f32(w < 0.5f ? a + w * d : b - d * (1.f - w));
+    v.e[i] = Tag::from_f32(fabsf(w) < 0.5f ? a + w * d : b - d * (1.f - w));
   }
 }
 

@@ -43,6 +43,7 @@ struct AttnParams {
   void* out;
   uint16_t* ws_o;  // [n_splits][rows >= ws_row0][Dh] normalised partial outputs / row scale, fp16 in [-1, 1]
   float* ws_ml;    // [n_splits][rows >= ws_row0][4]  softmax reference (log2 domain), sum, row scale, unused
+  uint32_t* ws_ctr;  // arrival counters of the in-kernel merge: 8 regions (one per XCD), zero between calls
   int64_t qs_b, qs_h, qs_t;
   int64_t os_b, os_h, os_t;
   int64_t L;
@@ -55,6 +56,8 @@ struct AttnParams {
   int group;        // query heads per kv head, H / Hkv
   int members;      // workgroups that share one K/V stream: group * q_tiles
   int unit_splits;  // units_whole + (B * Hkv - units_whole) * n_splits
+  int merge;        // split parts are merged by the main kernel (all workgroups of a unit on one XCD)
+  int merge_wait;   // ticks of the 100 MHz counter a part waits for the others before it gives up its share (0: none)
   float scale_log2;  // softmax scale * log2(e), applied to the raw logits in fp32
   // optional per (batch, head, token) output gate, element type (src/model/attn.py:117-119): either
   // given (sigmoid applied), or computed here from the module's input and gate_proj.weight
@@ -63,8 +66,9 @@ struct AttnParams {
   const void* gate_x;   // x[b, t, 0:H], channel stride 1, element strides gx_b / gx_t (null: no projection here)
   const void* gate_w;   // gate_proj.weight [H, H] row-major (out, in), element type
   int64_t gx_b, gx_t;
-  // measurement aid (null = off): every workgroup of the main kernel leaves its duration as
-  // (shader-clock cycles, ticks of the constant 100 MHz counter) at [2 * linear workgroup id]
+  // measurement library only (the product's kernels hold no code that reads it): every workgroup
+  // of the main kernel leaves its duration as (shader-clock cycles, ticks of the constant 100 MHz
+  // counter) at [2 * linear workgroup id]
   uint64_t* clock_out;
   int q_dma;            // 128-query workgroups fetch their Q tile by DMA (row offsets fit 32 bits)
 };
@@ -95,7 +99,7 @@ hipError_t launch_attn_ring_f16_64(const AttnParams& p, int ksplit, hipStream_t 
 // fp32 caches: plain vector-ALU kernel, one pass, no context splitting
 hipError_t launch_attn_ring_f32(const AttnParams& p, int Dh, hipStream_t stream);
 hipError_t launch_attn_combine(const AttnParams& p, int Dh, int dtype, hipStream_t stream);
-// Measurement aid (stream_probe.hip): the 256-token-frame tile stream without the arithmetic.
+// Measurement library only (stream_probe.hip): the 256-token-frame tile stream without the arithmetic.
 hipError_t launch_stream_probe(const void* src, int workgroups, int tiles, int share, hipStream_t stream);
 
 }  // namespace we

@@ -44,14 +44,48 @@ def _stream_ptr(dev: torch.device) -> int:
     return torch.cuda.current_stream(dev).cuda_stream
 
 
-def _call(dev: torch.device, fn, *args):
-    """Call a library entry point with the tensors' device current: the library configures and
-    launches its kernels on the device that is current when it is called (per-device LDS limits,
+_initialised = set()   # (library handle id, device index) pairs whose one-time set-up has run
+
+
+def init(device=None, probe: bool = False) -> None:
+    """One-time set-up of a device for the library (``we_init``): kernel LDS limits, the static
+    scratch buffer's address, and a small probe launch that checks the workgroup -> XCD mapping the
+    in-kernel merge of split-context parts relies on.  Synchronises the device once.  Every wrapper
+    here does it on first use; code that captures HIP graphs without an eager warm-up call calls
+    this first (the set-up cannot run under capture)."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    if dev.index is None:
+        dev = torch.device("cuda", torch.cuda.current_device())
+    lib = _capi.probe_lib() if probe else _capi.lib()
+    key = (id(lib), dev.index)
+    if key in _initialised:
+        return
+    if torch.cuda.is_current_stream_capturing():
+        raise RuntimeError("world_engine_amd: the first call on a device cannot be made under graph capture; call "
+                           "world_engine_amd.ops.init(device) (or make one eager call) beforehand")
+    with torch.cuda.device(dev):
+        _capi.check(lib.we_init(), "we_init")
+    _initialised.add(key)
+
+
+def _call(dev: torch.device, fn, *args, probe: bool = False):
+    """Call a library entry point with the tensors' device current: the library launches its
+    kernels on the device that is current when it is called and keeps per-device facts (LDS limits,
     the static scratch buffer's address).  No overhead when it already is."""
+    if (id(_capi.probe_lib() if probe else _capi.lib()), dev.index) not in _initialised:
+        init(dev, probe)
     if dev.index == torch.cuda.current_device():
         return fn(*args)
     with torch.cuda.device(dev):
         return fn(*args)
+
+
+def new_workspace(n_bytes: int, dev: torch.device) -> Tensor:
+    """A split-context workspace as the library wants to find it: the arrival counters at its start
+    zero (every call leaves them zero again), the rest uninitialised."""
+    ws = torch.empty(n_bytes, dtype=torch.uint8, device=dev)
+    ws[: _capi.WE_WS_COUNTER_BYTES].zero_()
+    return ws
 
 
 def _bhtd_strides(t: Tensor, what: str):
@@ -172,10 +206,23 @@ def attn_workspace_bytes(B: int, H: int, Hkv: int, T: int, Dh: int, L: int, n_sp
     return int(_capi.lib().we_attn_workspace_bytes(B, H, Hkv, T, Dh, L, n_splits, q_tile))
 
 
+def attn_plan(B: int, H: int, Hkv: int, T: int, Dh: int, L: int, n_splits: int = 0, q_tile: int = 0,
+              compute_units: int = 0, xcd_merge: Optional[bool] = True, two_pass: bool = False) -> dict:
+    """What the library would do with an attention call of these sizes (``we_attn_plan``; launches
+    nothing, needs no GPU when ``compute_units`` is given).  ``xcd_merge=None``: as the current
+    device's set-up found it, i.e. what a call on that device will really do."""
+    out = (ctypes.c_int32 * _capi.WE_PLAN_FIELDS)()
+    code = _capi.lib().we_attn_plan(B, H, Hkv, T, Dh, L, n_splits, q_tile | (_capi.WE_SPLIT_TWO_PASS if two_pass else 0),
+                                    compute_units, -1 if xcd_merge is None else int(bool(xcd_merge)), out)
+    _capi.check(code, "we_attn_plan")
+    return {"q_tile": out[0], "n_splits": out[1], "units_whole": out[2], "merge_in_kernel": bool(out[3]),
+            "workgroups": out[4], "compute_units": out[5]}
+
+
 def attn_ring(q: Tensor, kv: Tensor, written: Tensor, t_pos: Tensor, L: int, dilation: int,
               scale: Optional[float] = None, n_splits: int = 0, q_tile: int = 0,
               out: Optional[Tensor] = None, workspace: Optional[Tensor] = None,
-              token_major_out: bool = True, clocks: Optional[Tensor] = None) -> Tensor:
+              token_major_out: bool = True, clocks: Optional[Tensor] = None, two_pass: bool = False) -> Tensor:
     """Attention of one frame's queries over the visible part of the ring buffer.
 
     Replaces ``make_block_mask`` + ``flex_attention`` (``src/model/kv_cache.py:141-144``,
@@ -183,8 +230,12 @@ def attn_ring(q: Tensor, kv: Tensor, written: Tensor, t_pos: Tensor, L: int, dil
     ``[2,B,Hkv,L+T,Dh]``, ``written`` ``[L+T]`` bool, ``t_pos`` int64 with the frame index at
     element 0.  Returns ``[B,H,T,Dh]``; with ``token_major_out`` its memory is ``[B,T,H,Dh]`` so
     that ``y.transpose(1, 2).reshape(B, T, H*Dh)`` is a view (``src/patch_model.py:139``).
-    ``clocks`` (int64 device tensor, measurement aid): per workgroup of the main kernel its duration
-    in shader-clock cycles and in ticks of the constant 100 MHz counter (``we_attn_ring_fwd_clocked``).
+    ``workspace`` (split-context scratch, ``new_workspace``) is allocated when not given.
+    ``two_pass`` merges split-context parts with the second kernel even where the main kernel would
+    do it itself (same bits; for comparisons).
+    ``clocks`` (int64 device tensor): the call goes through the measurement library
+    (``libwe_probe.so``, ``we_attn_ring_fwd_clocked``), which also leaves, per workgroup of the main
+    kernel, its duration in shader-clock cycles and in ticks of the constant 100 MHz counter.
     """
     dev = _need_device(q, kv, written, t_pos)
     if q.dim() != 4:
@@ -200,10 +251,13 @@ def attn_ring(q: Tensor, kv: Tensor, written: Tensor, t_pos: Tensor, L: int, dil
     if t_pos.dtype != torch.long or t_pos.numel() < 1:
         raise RuntimeError("t_pos must be a non-empty int64 tensor")
     scale = 1.0 / math.sqrt(Dh) if scale is None else float(scale)
-    lib = _capi.lib()
-    ws_bytes = int(lib.we_attn_workspace_bytes(B, H, Hkv, T, Dh, L, n_splits, q_tile))
+    lib = _capi.probe_lib() if clocks is not None else _capi.lib()
+    if two_pass:
+        q_tile |= _capi.WE_SPLIT_TWO_PASS
+    with torch.cuda.device(dev):      # (the size depends on the device's compute-unit count)
+        ws_bytes = int(lib.we_attn_workspace_bytes(B, H, Hkv, T, Dh, L, n_splits, q_tile))
     if ws_bytes and (workspace is None or workspace.numel() * workspace.element_size() < ws_bytes):
-        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        workspace = new_workspace(ws_bytes, dev)
     if out is None:
         if token_major_out:
             out = torch.empty((B, T, H, Dh), dtype=q.dtype, device=dev).transpose(1, 2)
@@ -219,7 +273,8 @@ def attn_ring(q: Tensor, kv: Tensor, written: Tensor, t_pos: Tensor, L: int, dil
     if clocks is not None:
         if clocks.dtype != torch.int64 or not clocks.is_contiguous() or clocks.device != dev:
             raise RuntimeError("clocks must be a contiguous int64 tensor on q's device")
-        code = _call(dev, lib.we_attn_ring_fwd_clocked, *common, clocks.data_ptr(), clocks.numel(), _stream_ptr(dev))
+        code = _call(dev, lib.we_attn_ring_fwd_clocked, *common, clocks.data_ptr(), clocks.numel(), _stream_ptr(dev),
+                     probe=True)
         _capi.check(code, "we_attn_ring_fwd_clocked")
     else:
         code = _call(dev, lib.we_attn_ring_fwd, *common, _stream_ptr(dev))
@@ -259,14 +314,14 @@ def attn_ring_static(q: Tensor, kv: Tensor, written: Tensor, t_pos: Tensor, L: i
 
 
 def stream_probe(buf: Tensor, workgroups: int, tiles: int, share: int = 1) -> None:
-    """Measurement aid (``we_stream_probe``): ``workgroups`` workgroups each stream ``tiles`` 16-KB
+    """Measurement library (``libwe_probe.so``, ``we_stream_probe``): ``workgroups`` workgroups each stream ``tiles`` 16-KB
     tiles of ``buf`` into LDS the way the attention kernel fetches K/V tiles at 256-token frames,
     ``share`` workgroups per region, and compute nothing.  Time the launches from outside."""
     dev = _need_device(buf)
     if not buf.is_contiguous():
         raise RuntimeError("buf must be contiguous")
-    code = _call(dev, _capi.lib().we_stream_probe, buf.data_ptr(), buf.numel() * buf.element_size(), workgroups, tiles,
-                 share, _stream_ptr(dev))
+    code = _call(dev, _capi.probe_lib().we_stream_probe, buf.data_ptr(), buf.numel() * buf.element_size(), workgroups,
+                 tiles, share, _stream_ptr(dev), probe=True)
     _capi.check(code, "we_stream_probe")
 
 
@@ -335,9 +390,10 @@ def rope_kv_attn(q: Tensor, k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor],
     t_pos, y_pos, x_pos, ps = _pos_triplet(pos_ids, B, T, True)
     scale = 1.0 / math.sqrt(Dh) if scale is None else float(scale)
     lib = _capi.lib()
-    ws_bytes = int(lib.we_attn_workspace_bytes(B, H, Hkv, T, Dh, L, n_splits, q_tile))
+    with torch.cuda.device(dev):
+        ws_bytes = int(lib.we_attn_workspace_bytes(B, H, Hkv, T, Dh, L, n_splits, q_tile))
     if ws_bytes and (workspace is None or workspace.numel() * workspace.element_size() < ws_bytes):
-        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        workspace = new_workspace(ws_bytes, dev)
     q_rot = torch.empty((B, H, T, Dh), dtype=q.dtype, device=dev)
     if out is None:
         if token_major_out:
@@ -415,8 +471,9 @@ def qkv_rope_kv_attn(x: Tensor, w_qkv: Tensor, n_heads: int, n_kv_heads: int, po
                      _dtype_code(kv), extras, _stream_ptr(dev))
         _capi.check(code, "we_qkv_rope_kv_store")
         return None, q_rot, v_raw
-    ws_bytes = int(lib.we_attn_workspace_bytes(B, H, Hkv, T, Dh, L, n_splits, q_tile))
-    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+    with torch.cuda.device(dev):
+        ws_bytes = int(lib.we_attn_workspace_bytes(B, H, Hkv, T, Dh, L, n_splits, q_tile))
+    workspace = new_workspace(ws_bytes, dev) if ws_bytes else None
     out = torch.empty((B, T, H, Dh), dtype=x.dtype, device=dev).transpose(1, 2)
     code = _call(dev, lib.we_qkv_rope_kv_attn_fwd, *head, out.data_ptr(), _bhtd_strides(out, "out"),
                  workspace.data_ptr() if ws_bytes else None, ws_bytes,
