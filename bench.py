@@ -355,12 +355,14 @@ def run_gpu(cfg_id, c, args, torch, ro, wea, ops):
     # ---- shader clock inside the main kernel: cycles against the constant 100 MHz counter, per workgroup ----
     if not args.eager:
         try:
-            clocks = torch.zeros(2 * 65536, dtype=torch.int64, device=dev)
+            clocks = torch.zeros(_capi.WE_CLOCK_SLOTS * 65536, dtype=torch.int64, device=dev)
             for _ in range(60):                       # back to back, so the board sits at its sustained clock
                 ops.attn_ring(q_rot, layer0.kv, layer0.written, pos["t_pos"], layer0.L, 1, n_splits=args.n_splits,
                               q_tile=q_tile, out=out, workspace=ws, clocks=clocks)
             torch.cuda.synchronize()
-            ck = clocks.view(-1, 2).cpu()
+            rec = clocks.view(-1, _capi.WE_CLOCK_SLOTS).cpu()
+            rec = rec[rec[:, 1] > 0]
+            ck = rec[:, :2]
             ck = ck[ck[:, 1] > 0].double()
             ghz = (ck[:, 0] / (ck[:, 1] * 10.0)).tolist()          # cycles per 10 ns tick
             wg_us = (ck[:, 1] / 100.0).tolist()
@@ -372,6 +374,19 @@ def run_gpu(cfg_id, c, args, torch, ro, wea, ops):
                                             "clock per workgroup over the same interval on the constant 100 MHz counter"}
             log(f"[bench] shader clock inside attn_ring_kernel: {roof['shader_clock']['ghz_median']} GHz "
                 f"(workgroups run {roof['shader_clock']['workgroup_us_median']} us, longest {roof['shader_clock']['workgroup_us_max']} us)")
+            # where a workgroup's time goes: stage stamps of its first thread (us since its start), median over
+            # the workgroups and for the workgroup that ended last
+            names = ["slot_list", "first_k_tile", "loop_left", "pair_merged", "stored", "own_rows_acked", "all_rows_acked",
+                     "counted_in", "shares_known", "merged"]
+            stages = rec[:, 2:2 + len(names)].double() / 100.0
+            last = int(rec[:, 1].argmax())
+            roof["workgroup_timeline_us"] = {
+                "median": {n: round(percentile(stages[:, i][stages[:, i] > 0].tolist() or [0.0], 0.5), 2) for i, n in enumerate(names)},
+                "last_to_end": {n: round(float(stages[last, i]), 2) for i, n in enumerate(names)},
+                "what": "clocked instantiation (measurement library): us from a workgroup's start to each stage; stages after "
+                        "'stored' exist only when the kernel merges context parts itself"}
+            log(f"[bench] workgroup timeline (median): {roof['workgroup_timeline_us']['median']}")
+            log(f"[bench] workgroup timeline (last to end): {roof['workgroup_timeline_us']['last_to_end']}")
             del clocks
         except Exception as e:                      # noqa: BLE001 - a missing figure, not a failed benchmark
             roof["shader_clock"] = None

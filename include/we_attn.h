@@ -185,8 +185,11 @@ int we_attn_plan(int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64
  *                        The parts are merged by the main kernel itself - by whichever workgroup
  *                        of a query tile finishes last, through the L2 of the XCD that all parts
  *                        of a unit are placed on - when the device passed we_init's XCD check and
- *                        both the split and the unsplit unit counts are multiples of 8; otherwise
- *                        by a second kernel.  Both routes give the same bits.
+ *                        both the split and the unsplit unit counts are multiples of 8 (at most
+ *                        16 parts); otherwise by a second kernel.  Both routes give the same
+ *                        bits.  The first route relies on the placement we_init checked on the
+ *                        null stream: a stream that restricts the CUs a kernel may use (a CU
+ *                        mask) can place workgroups differently - pass WE_SPLIT_TWO_PASS there.
  *   q_tile               queries per workgroup: 0 = choose automatically, or 128 / 256;
  *                        optionally | WE_SPLIT_TWO_PASS.
  *   scale                softmax scale (> 0); the reference uses 1/sqrt(Dh).

@@ -19,14 +19,20 @@ extern "C" {
 
 /*
  * we_attn_ring_fwd that also records how long every workgroup of the main kernel ran, on two
- * clocks.  clocks[2 * w] receives workgroup w's duration in shader-clock cycles, clocks[2 * w + 1]
- * the same interval in ticks of the device's constant 100 MHz counter, w being the linear
- * workgroup id of the launch; their ratio is the shader clock the kernel actually ran at (boards
- * lower it under their power limit).  clocks_len = number of uint64 elements available; at least
- * 2 * (workgroups of the launch) or WE_ERR_WORKSPACE is returned; entries of workgroups that own
- * no work stay untouched (zero them beforehand).  bf16 / f16 only.  Everything else as
- * we_attn_ring_fwd; the output has the same bits.
+ * clocks, and when it passed the kernel's stages.  Workgroup w (the linear workgroup id of the
+ * launch) owns clocks[WE_CLOCK_SLOTS * w ...]: [0] its duration in shader-clock cycles, [1] the
+ * same interval in ticks of the device's constant 100 MHz counter (their ratio is the shader
+ * clock the kernel actually ran at; boards lower it under their power limit), [2 + s] the ticks
+ * from its start to stage s as seen by its first thread: 0 slot list built, 1 first K tile in
+ * LDS, 2 tile loop left, 3 wavefront pair merged, 4 (partial) results stored, and for workgroups
+ * that merge context parts themselves 5 own partial rows acknowledged, 6 every wavefront's, 7
+ * counted in, 8 shares known, 9 merged; [2 + 11] the shares it merged (bit mask).
+ * clocks_len = number of uint64 elements available; at least WE_CLOCK_SLOTS * (workgroups of the
+ * launch) or WE_ERR_WORKSPACE is returned; entries of workgroups that own no work, and of stages
+ * a workgroup does not pass, stay untouched (zero them beforehand).  bf16 / f16 only.  Everything
+ * else as we_attn_ring_fwd; the output has the same bits.
  */
+#define WE_CLOCK_SLOTS 16
 int we_attn_ring_fwd_clocked(const void* q, const int64_t q_strides[3],
                              const void* kv, const uint8_t* written, const int64_t* t_pos,
                              void* out, const int64_t out_strides[3],

@@ -235,3 +235,52 @@ def test_module_with_fused_neighbours(gpu_device):
         assert d1 <= 2e-2 * max(1.0, ya.float().abs().max().item()) and d2 <= 3e-2 * max(1.0, scale), (t, d1, d2)
         for li in range(2):
             assert_ulp_close(caches[1].layers[li].kv, caches[0].layers[li].kv, f"layer {li} cache t={t}", ulps=2 if li else 1)
+
+
+def test_eager_loop_reuses_its_per_layer_buffers(gpu_device):
+    """A serving loop in eager mode: with ``reuse_buffers`` the rotated q, the output and the
+    split-context workspace of a layer are allocated on its first call and used again by every
+    later one - the allocator's event count stays flat over 50 frames - and the results are those
+    of a twin cache whose calls allocate afresh.  Moving the cache drops the buffers."""
+    dev = gpu_device
+    B, H, Hkv, T, Dh, n = 1, 8, 8, 128, 128, 4
+    p = Pair(dev, torch.bfloat16, B=B, H=H, Hkv=Hkv, T=T, Dh=Dh, n_slots=n, n_layers=2, cfg_id=63)
+    twin = Pair(dev, torch.bfloat16, B=B, H=H, Hkv=Hkv, T=T, Dh=Dh, n_slots=n, n_layers=2, cfg_id=63)
+    p.set_frozen(False)
+    twin.set_frozen(False)
+    assert ops.attn_workspace_bytes(B, H, Hkv, T, Dh, n * T) > 0, "the case must need a workspace"
+    frames = []
+    for t in range(50):
+        q, k, v, pos = p.inputs(t % 7)
+        pos = ro.synth_pos_ids(t, B, T, p.W)
+        frames.append((q.to(dev), k.to(dev), v.to(dev), to_dev(pos, dev)))
+    torch.cuda.synchronize()
+    events = None
+    for t, (q, k, v, pos) in enumerate(frames):
+        outs = []
+        for layer in range(2):
+            y = p.hip.rope_upsert_attend(q, k, v, pos, p.rope, layer, reuse_buffers=True)
+            ref = twin.hip.rope_upsert_attend(q, k, v, pos, twin.rope, layer)
+            assert torch.equal(y, ref), f"frame {t} layer {layer}: reused buffers change the result"
+            outs.append(y.data_ptr())
+        if t == 0:
+            first_ptrs = outs
+        assert outs == first_ptrs and outs[0] != outs[1], "every layer keeps its own output buffer"
+        del y, ref
+        if t == 1:                               # steady state from the second frame on
+            events = _alloc_events_of_reusing_calls(p, frames[1])
+    assert events == 0, f"{events} allocations per frame in the steady state of the reusing path"
+    assert len(p.hip.layers[0]._call_buffers) == 1
+    p.hip.to(dev, torch.bfloat16)
+    assert len(p.hip.layers[0]._call_buffers) == 0, "moving or casting the cache drops the call buffers"
+
+
+def _alloc_events_of_reusing_calls(p, frame):
+    """Allocator events (torch.cuda.memory_stats) caused by one more frame through the reusing path."""
+    q, k, v, pos = frame
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_stats()["allocation.all.allocated"]
+    for layer in range(2):
+        p.hip.rope_upsert_attend(q, k, v, pos, p.rope, layer, reuse_buffers=True)
+    torch.cuda.synchronize()
+    return torch.cuda.memory_stats()["allocation.all.allocated"] - before

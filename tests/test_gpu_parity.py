@@ -396,10 +396,11 @@ def test_clocked_entry_point_same_output_and_plausible_clocks(gpu_device):
         (q_o, k_all, v_all, mask), (q_h, ring) = p.store(q, k, v, pos)
     plain = p.attend(q_h, ring, n_splits=2)
     assert_attn_close(plain, ro.attention_fp32(q_o, k_all, v_all, mask), "plain")
-    clocks = torch.zeros(2 * 1024, dtype=torch.int64, device=gpu_device)
+    clocks = torch.zeros(_capi.WE_CLOCK_SLOTS * 1024, dtype=torch.int64, device=gpu_device)
     timed = p.attend(q_h, ring, n_splits=2, clocks=clocks)
     assert_bits_equal(timed, plain, "clocked output")
-    c = clocks.view(-1, 2).cpu()
+    rec = clocks.view(-1, _capi.WE_CLOCK_SLOTS).cpu()
+    c = rec[:, :2]
     c = c[c[:, 0] != 0]
     _say(f"clocked: {c.shape[0]} workgroups, cycles {c[:4, 0].tolist()} ticks {c[:4, 1].tolist()}")
     # 1 query tile x 2 query heads per kv head x (2 kv heads x 2 context parts); grid slots past

@@ -21,6 +21,7 @@ WE_STATIC_SCRATCH_BYTES = 32 << 20
 WE_WS_COUNTER_BYTES = 16384
 WE_SPLIT_TWO_PASS = 0x10000
 WE_PLAN_FIELDS = 6
+WE_CLOCK_SLOTS = 16
 WE_ERR_SCRATCH_LIMIT = -7
 WE_ERR_NOT_READY = -8
 

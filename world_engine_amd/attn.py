@@ -235,7 +235,7 @@ class RingAttn(nn.Module):
         if self.gated_attn:
             extras.update(gate_x=x[..., : self.n_heads], gate_w=self.gate_proj.weight)
         y, v = kv_cache.qkv_rope_upsert_attend(x, self.qkv_proj.weight, self.n_heads, pos_ids, self.rope,
-                                               self.layer_idx, want_v=first, **extras)
+                                               self.layer_idx, want_v=first, reuse_buffers=True, **extras)
         if first:
             v1 = v
         return self.out_proj(y.transpose(1, 2).reshape(B, T, -1)), v1
@@ -284,7 +284,8 @@ class RingAttn(nn.Module):
         # RoPE(q), RoPE(k), cache write (one launch) and attention over the ring (one or two), all
         # behind one library call; a cache without it gets the reference's sequence of calls
         if hasattr(kv_cache, "rope_upsert_attend"):
-            y = kv_cache.rope_upsert_attend(q, k, v, pos_ids, self.rope, self.layer_idx, **extras)
+            # (y lives in the layer's own buffer until this layer's next call; out_proj below reads it now)
+            y = kv_cache.rope_upsert_attend(q, k, v, pos_ids, self.rope, self.layer_idx, reuse_buffers=True, **extras)
         else:
             q, k_all, v_all, ring = kv_cache.rope_upsert(q, k, v, pos_ids, self.rope, self.layer_idx)
             y = ring_attention(q, k_all, v_all, ring, enable_gqa=self.enable_gqa)

@@ -6,19 +6,22 @@
 #include "attn_mma.h"
 #include "we_kernels.h"
 
+
 namespace we {
 
-// 16-byte load of partial results.  L2: the load must not be served from this CU's vector L1
-// (the partials were written by other CUs of the same XCD a moment ago and live in its L2).
-template <bool L2>
-__device__ __forceinline__ u32x4_t load_partial16(const void* base, int64_t byte_off) {
-  if (L2) {
+// 16-byte load of partial results at base + lane_off + uniform_off.  L2: the load must not be
+// served from this CU's vector L1 (the partials were written by other CUs of the same XCD a moment
+// ago and live in its L2); its offsets are 32-bit (the host keeps the workspace of a call that
+// merges this way below 4 GiB) and the uniform part travels in a scalar register.
+template <bool L2, typename Off>
+__device__ __forceinline__ u32x4_t load_partial16(const void* base, Off lane_off, Off uniform_off) {
+  if constexpr (L2) {
     const __amdgpu_buffer_rsrc_t rs =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)0xffffffffu, 0x00020000);
-    // (the host keeps the workspace of a call that merges this way below 4 GiB)
-    return __builtin_amdgcn_raw_buffer_load_b128(rs, (int)(uint32_t)byte_off, 0, 16 /* sc1: miss the vector L1 */);
+    return __builtin_amdgcn_raw_buffer_load_b128(rs, (int)lane_off, (int)uniform_off, 16 /* sc1: miss the vector L1 */);
+  } else {
+    return *reinterpret_cast<const u32x4_t*>(static_cast<const unsigned char*>(base) + lane_off + uniform_off);
   }
-  return *reinterpret_cast<const u32x4_t*>(static_cast<const unsigned char*>(base) + byte_off);
 }
 
 // Every split left, per query row, its normalised output as fp16 values times a row scale r_s, its
@@ -31,20 +34,26 @@ struct PartialBatch {
   f16x8_t ov[8];
 };
 
-// Requests splits [s0, s0 + 8) of workspace row `wrow` (query row - ws_row0; `rows` = the
-// workspace's row count), columns [8 dg, 8 dg + 8).
-template <int DH, bool L2>
-__device__ __forceinline__ void load_batch(PartialBatch& pb, const AttnParams& p, int64_t rows, int64_t wrow, int dg, int s0) {
+// Requests splits [s0, s0 + 8) of one item: ml_off / o_off are the byte offsets of split 0's record
+// and of its 8 columns in the two workspace areas, ml_step / o_step the distance between splits.
+// Off is uint32_t for the in-kernel merge and int64_t for the second-pass kernel.  (The in-kernel
+// merge runs once per launch, straight out of memory and on one wavefront's issue rate: every
+// instruction of address arithmetic saved here is time off the end of the kernel.)
+template <bool L2, typename Off>
+__device__ __forceinline__ void load_batch(PartialBatch& pb, const AttnParams& p, Off ml_off, Off o_off, Off ml_step,
+                                           Off o_step, int s0) {
+  Off ml_s = (Off)s0 * ml_step, o_s = (Off)s0 * o_step;   // uniform
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     if (s0 + j < p.n_splits) {  // (uniform: a request is 16 cycles of the CU's address path whether wanted or not)
-      const int64_t r = (int64_t)(s0 + j) * rows + wrow;
-      pb.ml[j] = __builtin_bit_cast(f32x4_t, load_partial16<L2>(p.ws_ml, r * 16));
-      pb.ov[j] = __builtin_bit_cast(f16x8_t, load_partial16<L2>(p.ws_o, (r * DH + dg * 8) * 2));
+      pb.ml[j] = __builtin_bit_cast(f32x4_t, load_partial16<L2, Off>(p.ws_ml, ml_off, ml_s));
+      pb.ov[j] = __builtin_bit_cast(f16x8_t, load_partial16<L2, Off>(p.ws_o, o_off, o_s));
     } else {
       pb.ml[j] = f32x4_t{-INFINITY, 0.f, 0.f, 0.f};
       pb.ov[j] = f16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
     }
+    ml_s += ml_step;
+    o_s += o_step;
   }
 }
 
@@ -87,16 +96,19 @@ __device__ __forceinline__ void finish_item(const AttnParams& p, const float (&a
   *reinterpret_cast<frag_t*>(dst) = y;
 }
 
-// One output item, any number of splits.
-template <typename M, int DH, bool L2>
-__device__ __forceinline__ void merge_item(const AttnParams& p, int64_t rows, int64_t wrow, int b, int h, int t, int dg) {
+// One output item, any number of splits: ml_off / o_off / ml_step / o_step as for load_batch, query
+// row (b, h, t), columns [8 dg, 8 dg + 8).
+template <typename M, bool L2, typename Off>
+__device__ __forceinline__ void merge_item(const AttnParams& p, Off ml_off, Off o_off, Off ml_step, Off o_step, int b,
+                                           int h, int t, int dg) {
   float mmax = -INFINITY, den = 0.f;
   float acc[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+#pragma nounroll
   for (int s0 = 0; s0 < p.n_splits; s0 += 8) {
     PartialBatch pb;
-    load_batch<DH, L2>(pb, p, rows, wrow, dg, s0);
+    load_batch<L2, Off>(pb, p, ml_off, o_off, ml_step, o_step, s0);
     accumulate_batch(pb, p.n_splits - s0, mmax, den, acc);
   }
   finish_item<M>(p, acc, den, b, h, t, dg);

@@ -187,8 +187,12 @@ inline int prepare_attn(const void* q, const int64_t* q_strides, const void* kv,
   p.group = H / Hkv;
   p.members = p.group * p.q_tiles;
   p.unit_splits = pl.units_whole + (B * Hkv - pl.units_whole) * pl.n_splits;
+  if ((int64_t)B * H * T >= (1ll << 31)) pl.merge = 0;  // ... and rows with 32-bit indices
   p.merge = pl.merge;
-  p.merge_wait = pl.merge_wait;
+  p.merge_wait = pl.merge ? pl.merge_wait : 0;
+  p.ws_rows32 = (uint32_t)pl.ws_rows;
+  p.ws_row0_32 = (uint32_t)p.ws_row0;
+  p.share_items = (uint32_t)((pl.block_m * (Dh / 8) + pl.n_splits - 1) / pl.n_splits);
   p.scale_log2 = scale * 1.4426950408889634f;
   p.gate = nullptr; p.gs_b = p.gs_h = p.gs_t = 0;
   p.gate_x = nullptr; p.gate_w = nullptr; p.gx_b = p.gx_t = 0;

@@ -124,6 +124,13 @@ attn_ring_kernel(AttnParams p) {
   // shader-clock and constant-rate (100 MHz) counters at the workgroup's start
   const uint64_t clk0 = CLOCKED ? (uint64_t)__builtin_readcyclecounter() : 0;
   const uint64_t wall0 = CLOCKED ? (uint64_t)__builtin_amdgcn_s_memrealtime() : 0;
+  // CLOCKED: thread 0 also leaves the time (100 MHz ticks since the start) at which it passed each
+  // stage, at [kClockSlots * workgroup + 2 + stage]
+  const uint64_t wg_id = blockIdx.x + (uint64_t)gridDim.x * (blockIdx.y + (uint64_t)gridDim.y * blockIdx.z);
+  auto stamp = [&](int stage) __attribute__((always_inline)) {
+    if (CLOCKED && tid == 0)
+      p.clock_out[kClockSlots * wg_id + 2 + stage] = (uint64_t)__builtin_amdgcn_s_memrealtime() - wall0;
+  };
   const int qb = wave % QW;   // query block of this wavefront
   const int hb = wave / QW;   // key block of every tile it handles when KSPLIT == 2 (else 0)
 
@@ -213,6 +220,7 @@ attn_ring_kernel(AttnParams p) {
     if (lane == 0) vis[nvis] = p.n_slots;
     ++nvis;
   }
+  stamp(0);  // slot list built
   // tiles per slot; the last one of a slot holds t_last of its 64 keys when T % 64 != 0
   const int tps = (p.T + BN - 1) / BN;
   const int t_last = p.T - (tps - 1) * BN;
@@ -562,6 +570,7 @@ attn_ring_kernel(AttnParams p) {
     }
     dma_wait<(KA + 1) * NDMA>();
     __syncthreads();  // K(0) and the zeroed V slot (128-query shape: the Q tile, requested long before K(0)) are in LDS
+    stamp(1);  // first K tile landed
     if (KSPLIT == 2 && q_dma) {
       // row qb*32 + l32 of the tile, logical chunk 2*ks + hh: the K fragment's address arithmetic
       const int x = k_swz<DH>(l32);
@@ -659,6 +668,7 @@ attn_ring_kernel(AttnParams p) {
     if (j < ntile) { iteration(j, IntC<1>(), not_first); ++j; }
     if (j < ntile) { iteration(j, IntC<2>(), not_first); ++j; }
 
+    stamp(2);  // tile loop left
     // product of the last block: (ntile-1, 1) for full-tile wavefronts, (ntile-1, hb) otherwise
     {
       const int last = (ntile - 1) % NST;
@@ -726,6 +736,7 @@ attn_ring_kernel(AttnParams p) {
     }
   }
 
+  stamp(3);  // pair merged
   // ---- epilogue ----
   if (KSPLIT == 1 || hb == 0) {
   const int64_t rows = (int64_t)p.B * p.H * p.T - p.ws_row0;  // rows in the workspace
@@ -796,6 +807,7 @@ attn_ring_kernel(AttnParams p) {
     }
   }
   }  // (epilogue of the wavefronts that hold results)
+  stamp(4);  // results / partial results stored (requests issued)
 
   // ---- merge of the context parts, shared out among the workgroups that computed them ----
   // Every part has left its rows in the workspace with plain stores, i.e. in the L2 of the XCD that
@@ -814,7 +826,9 @@ attn_ring_kernel(AttnParams p) {
   //   word: bits 7:0 parts arrived, 15:8 parts departed, 31:16 shares given up by their owners
   if (merging) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    stamp(5);  // this wavefront's partial rows acknowledged
     __syncthreads();
+    stamp(6);  // every wavefront's
     volatile uint32_t* todo = reinterpret_cast<volatile uint32_t*>(smem + L::MISC_OFF);
     uint32_t* word = p.ws_ctr + xcd * host::kCtrPerXcd +
                      ((((unit - p.units_whole) >> 3) * p.group + hq_in) * p.q_tiles + qtile);
@@ -823,6 +837,8 @@ attn_ring_kernel(AttnParams p) {
     if (tid == 0) {
       uint32_t mine = 0;
       const uint32_t before = __hip_atomic_fetch_add(word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      if (CLOCKED) asm volatile("" ::"v"(before));
+      stamp(7);  // counted in
       if ((before & 0xffu) + 1u == parts) {
         mine = (before >> 16) | (1u << split);  // last in: its own share and those given up
       } else {
@@ -847,52 +863,41 @@ attn_ring_kernel(AttnParams p) {
       // round trip runs under the merge below.  The last to depart puts the word back to zero.
       departed = __hip_atomic_fetch_add(word, 0x100u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
-    __syncthreads();
-    uint32_t shares = (uint32_t)__builtin_amdgcn_readfirstlane((int)*todo);
-    const int64_t rows = (int64_t)p.B * p.H * p.T - p.ws_row0;
-    const int64_t wrow0 = ((int64_t)b * p.H + h) * p.T - p.ws_row0 + qtile * BM;
+    // (a bare barrier after the LDS write has landed: __syncthreads() would first wait for the
+    // departure's answer, which nobody needs before the end)
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    const uint32_t shares = (uint32_t)__builtin_amdgcn_readfirstlane((int)*todo);
+    stamp(8);  // shares known: every part is in (or this workgroup has given up)
+    if (CLOCKED && tid == 0) p.clock_out[kClockSlots * wg_id + 2 + 11] = shares;
+    // (row, 8 columns) items: 16 (Dh 128) or 8 consecutive lanes share a row, so requests cover
+    // whole rows.  Nothing is unrolled and all offsets are 32-bit (the host saw to it that they
+    // fit): this code runs once per launch, at one instruction per few cycles.  From four parts on
+    // a share is one item per thread.
+    constexpr uint32_t DG = DH / 8, N = BM * DG;
     const int t0 = qtile * BM;
-    constexpr int DG = DH / 8;
-    constexpr unsigned N = BM * DG;                       // (row, 8 columns) items of the tile
-    constexpr int MAXI = N / 2 / 512 > 0 ? N / 2 / 512 : 1;  // items per thread of the largest share (two parts)
-    for (; shares != 0u; shares &= shares - 1u) {
-      const unsigned k = (unsigned)__builtin_ctz(shares);
-      // 16 (Dh 128) or 8 consecutive lanes share a row: whole rows per request
-      const int lo = (int)(k * N / parts), hi = (int)((k + 1u) * N / parts);
-      if (p.n_splits <= 8) {
-        // one batch of loads per item; the next item's are requested before this item's arithmetic,
-        // so that a thread's items cost one trip to the L2 between them, not one each
-        PartialBatch cur, nxt;
-        int it = lo + tid;
-        bool ok = it < hi && t0 + it / DG < p.T;
-        if (ok) load_batch<DH, true>(cur, p, rows, wrow0 + it / DG, it % DG, 0);
-#pragma unroll
-        for (int i = 0; i < MAXI; ++i) {
-          const int itn = it + 512;
-          const bool okn = i + 1 < MAXI && itn < hi && t0 + itn / DG < p.T;
-          if (okn) load_batch<DH, true>(nxt, p, rows, wrow0 + itn / DG, itn % DG, 0);
-          if (ok) {
-            float mmax = -INFINITY, den = 0.f;
-            float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            accumulate_batch(cur, p.n_splits, mmax, den, acc);
-            finish_item<M>(p, acc, den, b, h, t0 + it / DG, it % DG);
-          }
-          cur = nxt;
-          it = itn;
-          ok = okn;
-        }
-      } else {
-        for (int it = lo + tid; it < hi; it += 512)
-          if (t0 + it / DG < p.T) merge_item<M, DH, true>(p, rows, wrow0 + it / DG, b, h, t0 + it / DG, it % DG);
+    const uint32_t wrow0 = (uint32_t)((b * p.H + h) * p.T + t0) - p.ws_row0_32;  // tile's first row in the workspace
+    const uint32_t ml_step = p.ws_rows32 * 16u, o_step = p.ws_rows32 * (uint32_t)(DH * 2);
+#pragma nounroll
+    for (uint32_t left = shares; left != 0u; left &= left - 1u) {
+      const uint32_t lo = (uint32_t)__builtin_ctz(left) * p.share_items;
+      const uint32_t hi = lo + p.share_items < N ? lo + p.share_items : N;
+#pragma nounroll
+      for (uint32_t it = lo + tid; it < hi; it += 512u) {
+        const uint32_t r = it / DG, dg = it % DG;
+        if (t0 + (int)r < p.T)
+          merge_item<M, true, uint32_t>(p, (wrow0 + r) * 16u, ((wrow0 + r) * DH + dg * 8u) * 2u, ml_step, o_step, b, h,
+                                        t0 + (int)r, (int)dg);
       }
     }
+    stamp(9);  // merged (requests issued)
     if (tid == 0 && ((departed >> 8) & 0xffu) + 1u == parts)
       __hip_atomic_store(word, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   }
   if (CLOCKED && tid == 0) {
-    const uint64_t wg = blockIdx.x + (uint64_t)gridDim.x * (blockIdx.y + (uint64_t)gridDim.y * blockIdx.z);
-    p.clock_out[2 * wg] = (uint64_t)__builtin_readcyclecounter() - clk0;
-    p.clock_out[2 * wg + 1] = (uint64_t)__builtin_amdgcn_s_memrealtime() - wall0;
+    p.clock_out[kClockSlots * wg_id] = (uint64_t)__builtin_readcyclecounter() - clk0;
+    p.clock_out[kClockSlots * wg_id + 1] = (uint64_t)__builtin_amdgcn_s_memrealtime() - wall0;
   }
 }
 

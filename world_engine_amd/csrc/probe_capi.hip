@@ -6,6 +6,8 @@
 #include "device_state.h"
 #include "we_kernels.h"
 
+static_assert(WE_CLOCK_SLOTS == we::kClockSlots, "header and kernels disagree on the clock record");
+
 extern "C" {
 
 int we_attn_ring_fwd_clocked(const void* q, const int64_t q_strides[3], const void* kv, const uint8_t* written,
@@ -26,7 +28,7 @@ int we_attn_ring_fwd_clocked(const void* q, const int64_t q_strides[3], const vo
                                         ds->xcd_merge, p, pl);
   if (rc != WE_OK) return rc;
   const size_t wgs = (size_t)(8 * p.q_tiles) * (size_t)p.group * (size_t)((p.unit_splits + 7) / 8);
-  if (clocks_len < 2 * wgs) return WE_ERR_WORKSPACE;
+  if (clocks_len < WE_CLOCK_SLOTS * wgs) return WE_ERR_WORKSPACE;
   p.clock_out = clocks;
   return we::host::launch_attn(p, pl, Dh, dtype, st);
 }

@@ -35,6 +35,9 @@ struct StoreParams {
   int64_t v1s_b, v1s_h, v1s_t;
 };
 
+// uint64 slots per workgroup of AttnParams::clock_out (measurement library only)
+constexpr int kClockSlots = 16;
+
 struct AttnParams {
   const void* q;
   const void* kv;
@@ -58,6 +61,10 @@ struct AttnParams {
   int unit_splits;  // units_whole + (B * Hkv - units_whole) * n_splits
   int merge;        // split parts are merged by the main kernel (all workgroups of a unit on one XCD)
   int merge_wait;   // ticks of the 100 MHz counter a part waits for the others before it gives up its share (0: none)
+  // in-kernel merge, precomputed so that the kernel's tail has no divisions and no 64-bit arithmetic:
+  uint32_t ws_rows32;    // rows of the workspace
+  uint32_t ws_row0_32;   // ws_row0
+  uint32_t share_items;  // (row, 8 columns) items of a query tile per share: ceil(queries per workgroup * Dh / 8 / n_splits)
   float scale_log2;  // softmax scale * log2(e), applied to the raw logits in fp32
   // optional per (batch, head, token) output gate, element type (src/model/attn.py:117-119): either
   // given (sigmoid applied), or computed here from the module's input and gate_proj.weight

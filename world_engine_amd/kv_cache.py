@@ -70,6 +70,20 @@ class LayerKVCache(nn.Module):
         offsets = torch.arange(T, dtype=torch.long)
         self.register_buffer("frame_offsets", offsets, persistent=False)
         self.register_buffer("current_idx", offsets + L, persistent=False)
+        # per-layer call buffers (rotated q, attention output, split-context workspace) of the eager
+        # path, sized on first use and dropped whenever the module is moved or cast
+        self._call_buffers = {}
+
+    def _apply(self, fn, *args, **kwargs):
+        self._call_buffers = {}
+        return super()._apply(fn, *args, **kwargs)
+
+    def _reusable(self, reuse: bool):
+        """The buffer dict for an eager call, or None where every call must own its tensors (under
+        torch.compile the opaque op allocates; under stream capture the graph owns what it captured)."""
+        if not reuse or torch.compiler.is_compiling() or torch.cuda.is_current_stream_capturing():
+            return None
+        return self._call_buffers
 
     def reset(self) -> None:
         self.kv.zero_()
@@ -119,10 +133,15 @@ class LayerKVCache(nn.Module):
                            is_frozen: bool, scale: Optional[float] = None, qk_norm_eps: float = 0.0,
                            v1: Optional[Tensor] = None, v_lamb: Optional[Tensor] = None,
                            gate: Optional[Tensor] = None, gate_x: Optional[Tensor] = None,
-                           gate_w: Optional[Tensor] = None) -> Tensor:
+                           gate_w: Optional[Tensor] = None, reuse_buffers: bool = False) -> Tensor:
         """``rope_upsert`` followed by the attention over the ring, as one library call
         (``src/model/attn.py:110-116`` of the reference from RoPE to ``flex_attention``).  Under
-        ``torch.compile`` the registered opaque op is used instead of the eager wrapper."""
+        ``torch.compile`` the registered opaque op is used instead of the eager wrapper.
+
+        ``reuse_buffers``: the rotated q, the output and the split-context workspace live in
+        per-layer tensors that the next eager call of this layer uses again, so a serving loop
+        allocates nothing after its first frame.  The returned tensor is then only valid until
+        that next call (the attention module consumes it at once); off by default."""
         if torch.compiler.is_compiling():
             s = float(scale) if scale is not None else float(q.shape[-1]) ** -0.5
             return torch.ops.world_engine_amd.rope_kv_attn(
@@ -130,16 +149,27 @@ class LayerKVCache(nn.Module):
                 rope.width, self.kv, self.written, self.L, self.pinned_dilation, bool(is_frozen), s,
                 float(qk_norm_eps), v1, v_lamb, gate, gate_x, gate_w)
         self._check(k, pos_ids, rope)
+        kept = self._reusable(reuse_buffers)
+        bufs = {}
+        if kept is not None:
+            B, H, T, Dh = q.shape
+            key = ("attn", B, H, k.shape[1], T, Dh, q.dtype, q.device)
+            if key not in kept:
+                ws_bytes = ops.attn_workspace_bytes(B, H, k.shape[1], T, Dh, self.L)
+                kept[key] = dict(q_rot=torch.empty((B, H, T, Dh), dtype=q.dtype, device=q.device),
+                                 out=torch.empty((B, T, H, Dh), dtype=q.dtype, device=q.device).transpose(1, 2),
+                                 workspace=ops.new_workspace(ws_bytes, q.device) if ws_bytes else None)
+            bufs = kept[key]
         return ops.rope_kv_attn(q, k, v, pos_ids, rope.cos, rope.sin, rope.height, rope.width, self.kv,
                                 self.written, self.L, self.pinned_dilation, is_frozen, scale,
                                 qk_norm_eps=qk_norm_eps, v1=v1, v_lamb=v_lamb, gate=gate, gate_x=gate_x,
-                                gate_w=gate_w)[0]
+                                gate_w=gate_w, **bufs)[0]
 
     def qkv_rope_upsert_attend(self, x: Tensor, w_qkv: Tensor, n_heads: int, pos_ids: Mapping[str, Tensor], rope,
                                is_frozen: bool, scale: Optional[float] = None, want_v: bool = False,
                                qk_norm_eps: float = 0.0, v1: Optional[Tensor] = None,
                                v_lamb: Optional[Tensor] = None, gate_x: Optional[Tensor] = None,
-                               gate_w: Optional[Tensor] = None) -> Tuple[Tensor, Optional[Tensor]]:
+                               gate_w: Optional[Tensor] = None, reuse_buffers: bool = False) -> Tuple[Tensor, Optional[Tensor]]:
         """``rope_upsert_attend`` with the module's merged q/k/v projection in front, as one
         library call (``src/patch_model.py:116-134`` from ``self.qkv_proj(x)`` to the attention
         output).  Returns ``(y, v)``: ``v`` (``want_v``) is the projected value rows before the
@@ -156,7 +186,7 @@ class LayerKVCache(nn.Module):
         y, _, v = ops.qkv_rope_kv_attn(x, w_qkv, n_heads, n_kv, pos_ids, rope.cos, rope.sin, rope.height, rope.width,
                                        self.kv, self.written, self.L, self.pinned_dilation, is_frozen, scale,
                                        want_v=want_v, qk_norm_eps=qk_norm_eps, v1=v1, v_lamb=v_lamb, gate_x=gate_x,
-                                       gate_w=gate_w)
+                                       gate_w=gate_w, buffers=self._reusable(reuse_buffers))
         return y, v
 
 

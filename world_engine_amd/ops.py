@@ -364,11 +364,12 @@ def rope_kv_attn(q: Tensor, k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor],
                  q_tile: int = 0, out: Optional[Tensor] = None, workspace: Optional[Tensor] = None,
                  token_major_out: bool = True, qk_norm_eps: float = 0.0, v1: Optional[Tensor] = None,
                  v_lamb: Optional[Tensor] = None, gate: Optional[Tensor] = None,
-                 gate_x: Optional[Tensor] = None, gate_w: Optional[Tensor] = None):
+                 gate_x: Optional[Tensor] = None, gate_w: Optional[Tensor] = None, q_rot: Optional[Tensor] = None):
     """``rope_kv_store`` followed by ``attn_ring`` in one library call (``we_rope_kv_attn_fwd``):
     the per-layer sequence of the reference from ``q, k = rope(q), rope(k)`` to the
     ``flex_attention`` call (``src/model/attn.py:110-116``), validated as a whole before the first
     launch.  Returns ``(out, q_rot)``; results are those of the two separate calls, bit for bit.
+    ``out``, ``workspace`` and ``q_rot`` (contiguous ``[B,H,T,Dh]``) are allocated when not given.
 
     Optional neighbours of the path done inside the kernels (``src/model/attn.py:105-109,117-119``):
     ``qk_norm_eps > 0`` RMS-normalises q and k rows first (``F.rms_norm`` without weight; torch's
@@ -394,7 +395,10 @@ def rope_kv_attn(q: Tensor, k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor],
         ws_bytes = int(lib.we_attn_workspace_bytes(B, H, Hkv, T, Dh, L, n_splits, q_tile))
     if ws_bytes and (workspace is None or workspace.numel() * workspace.element_size() < ws_bytes):
         workspace = new_workspace(ws_bytes, dev)
-    q_rot = torch.empty((B, H, T, Dh), dtype=q.dtype, device=dev)
+    if q_rot is None:
+        q_rot = torch.empty((B, H, T, Dh), dtype=q.dtype, device=dev)
+    elif tuple(q_rot.shape) != (B, H, T, Dh) or q_rot.dtype != q.dtype or q_rot.device != dev or not q_rot.is_contiguous():
+        raise RuntimeError("q_rot must be a contiguous [B, H, T, Dh] tensor of q's element type on q's device")
     if out is None:
         if token_major_out:
             out = torch.empty((B, T, H, Dh), dtype=q.dtype, device=dev).transpose(1, 2)
@@ -422,7 +426,8 @@ def qkv_rope_kv_attn(x: Tensor, w_qkv: Tensor, n_heads: int, n_kv_heads: int, po
                      L: int, dilation: int, is_frozen: bool, scale: Optional[float] = None, n_splits: int = 0,
                      q_tile: int = 0, attend: bool = True, want_v: bool = False, qk_norm_eps: float = 0.0,
                      v1: Optional[Tensor] = None, v_lamb: Optional[Tensor] = None, gate: Optional[Tensor] = None,
-                     gate_x: Optional[Tensor] = None, gate_w: Optional[Tensor] = None):
+                     gate_x: Optional[Tensor] = None, gate_w: Optional[Tensor] = None,
+                     buffers: Optional[dict] = None):
     """The module's merged q/k/v projection, RoPE, the cache write and (``attend``) the attention
     over the ring in one library call (``we_qkv_rope_kv_attn_fwd`` / ``we_qkv_rope_kv_store``):
     ``src/patch_model.py:116-134`` from ``self.qkv_proj(x)`` to the ``flex_attention`` call.  The
@@ -434,7 +439,9 @@ def qkv_rope_kv_attn(x: Tensor, w_qkv: Tensor, n_heads: int, n_kv_heads: int, po
     token-major memory, ``q_rot`` the rotated (normalised) queries, ``v`` (``want_v``) the projected
     value rows ``[B, Hkv, T, Dh]`` before the value blend - what the first layer returns as ``v1``.
     Projection rows are fp32 sums rounded once to the element type in a fixed order that differs
-    from a BLAS library's: they can differ from ``F.linear``'s in the last bit."""
+    from a BLAS library's: they can differ from ``F.linear``'s in the last bit.
+    ``buffers``: a dict the call keeps its ``q_rot`` / ``out`` / ``workspace`` tensors in and takes
+    them from next time (shapes permitting), for callers that step the same layer again and again."""
     dev = _need_device(x, w_qkv, kv, written, cos_table, sin_table, pos_ids["t_pos"])
     if x.dim() != 3 or x.stride(2) != 1:
         raise RuntimeError("x must be [B, T, d_model] with contiguous channels")
@@ -452,7 +459,15 @@ def qkv_rope_kv_attn(x: Tensor, w_qkv: Tensor, n_heads: int, n_kv_heads: int, po
     t_pos, y_pos, x_pos, ps = _pos_triplet(pos_ids, B, T, True)
     scale = 1.0 / math.sqrt(Dh) if scale is None else float(scale)
     lib = _capi.lib()
-    q_rot = torch.empty((B, H, T, Dh), dtype=x.dtype, device=dev)
+    def buf(name, make):
+        if buffers is None:
+            return make()
+        key = (name, B, H, Hkv, T, Dh, x.dtype, dev)
+        if key not in buffers:
+            buffers[key] = make()
+        return buffers[key]
+
+    q_rot = buf("q_rot", lambda: torch.empty((B, H, T, Dh), dtype=x.dtype, device=dev))
     proj = _capi.QkvProj()
     proj.x, proj.w, proj.d_model = x.data_ptr(), w_qkv.data_ptr(), d_model
     proj.x_strides = (ctypes.c_int64 * 2)(x.stride(0), x.stride(1))
@@ -473,8 +488,8 @@ def qkv_rope_kv_attn(x: Tensor, w_qkv: Tensor, n_heads: int, n_kv_heads: int, po
         return None, q_rot, v_raw
     with torch.cuda.device(dev):
         ws_bytes = int(lib.we_attn_workspace_bytes(B, H, Hkv, T, Dh, L, n_splits, q_tile))
-    workspace = new_workspace(ws_bytes, dev) if ws_bytes else None
-    out = torch.empty((B, T, H, Dh), dtype=x.dtype, device=dev).transpose(1, 2)
+    workspace = buf(("workspace", ws_bytes), lambda: new_workspace(ws_bytes, dev)) if ws_bytes else None
+    out = buf("out", lambda: torch.empty((B, T, H, Dh), dtype=x.dtype, device=dev).transpose(1, 2))
     code = _call(dev, lib.we_qkv_rope_kv_attn_fwd, *head, out.data_ptr(), _bhtd_strides(out, "out"),
                  workspace.data_ptr() if ws_bytes else None, ws_bytes,
                  B, H, Hkv, T, Dh, L, dilation, int(bool(is_frozen)), scale, n_splits, q_tile, _dtype_code(kv),
