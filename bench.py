@@ -178,11 +178,11 @@ def run_gpu(cfg_id, c, args, torch, ro, wea, ops):
     t_pos_all = torch.arange(nf, dtype=torch.long)[:, None, None].expand(nf, B, T).contiguous().to(dev)
 
     from world_engine_amd import _capi
-    q_tile = args.q_tile | (_capi.WE_SPLIT_TWO_PASS if args.two_pass else 0)
+    q_tile = args.q_tile
     ops.init(dev)
-    lib_plan = ops.attn_plan(B, H, Hkv, T, Dh, L, args.n_splits, args.q_tile, xcd_merge=None, two_pass=args.two_pass)
+    lib_plan = ops.attn_plan(B, H, Hkv, T, Dh, L, args.n_splits, args.q_tile)
     n_splits = lib_plan["n_splits"]
-    ws = ops.new_workspace(max(ops.attn_workspace_bytes(B, H, Hkv, T, Dh, L, args.n_splits, q_tile), 16), dev)
+    ws = torch.empty(max(ops.attn_workspace_bytes(B, H, Hkv, T, Dh, L, args.n_splits, q_tile), 16), dtype=torch.uint8, device=dev)
     out = torch.empty((B, T, H, Dh), dtype=dtype, device=dev).transpose(1, 2)
 
     def one_step(step_idx):
@@ -301,10 +301,7 @@ def run_gpu(cfg_id, c, args, torch, ro, wea, ops):
                 "frac": round(tflops / PEAK_BF16_TFLOPS, 4), "traffic": None}
     if not (args.n_splits or args.q_tile):
         roof["traffic"], roof["traffic_source"] = read_traffic(cfg_id)
-    roof.update({"kernel": "attn_ring_kernel" + (" + attn_combine_kernel" if n_splits > 1 and not lib_plan["merge_in_kernel"] else ""),
-                 "split_parts_merged": ("nothing split" if n_splits == 1 else
-                                        "inside attn_ring_kernel (last workgroup of a query tile, through its XCD's L2)"
-                                        if lib_plan["merge_in_kernel"] else "by attn_combine_kernel"),
+    roof.update({"kernel": "attn_ring_kernel" + (" + attn_combine_kernel" if n_splits > 1 else ""),
                  "workgroups": lib_plan["workgroups"], "compute_units": lib_plan["compute_units"],
                  "us_per_launch": round(attn_us, 3), "us_per_launch_p10": round(ast["p10"], 3),
                  "us_per_launch_p90": round(ast["p90"], 3), "launches_per_sample": iters,
@@ -376,15 +373,14 @@ def run_gpu(cfg_id, c, args, torch, ro, wea, ops):
                 f"(workgroups run {roof['shader_clock']['workgroup_us_median']} us, longest {roof['shader_clock']['workgroup_us_max']} us)")
             # where a workgroup's time goes: stage stamps of its first thread (us since its start), median over
             # the workgroups and for the workgroup that ended last
-            names = ["slot_list", "first_k_tile", "loop_left", "pair_merged", "stored", "own_rows_acked", "all_rows_acked",
-                     "counted_in", "shares_known", "merged"]
+            names = ["slot_list", "first_k_tile", "loop_left", "pair_merged", "stored"]
             stages = rec[:, 2:2 + len(names)].double() / 100.0
             last = int(rec[:, 1].argmax())
             roof["workgroup_timeline_us"] = {
                 "median": {n: round(percentile(stages[:, i][stages[:, i] > 0].tolist() or [0.0], 0.5), 2) for i, n in enumerate(names)},
                 "last_to_end": {n: round(float(stages[last, i]), 2) for i, n in enumerate(names)},
-                "what": "clocked instantiation (measurement library): us from a workgroup's start to each stage; stages after "
-                        "'stored' exist only when the kernel merges context parts itself"}
+                "what": "clocked instantiation (measurement library): us from a workgroup's start to each stage as its "
+                        "first thread passes it"}
             log(f"[bench] workgroup timeline (median): {roof['workgroup_timeline_us']['median']}")
             log(f"[bench] workgroup timeline (last to end): {roof['workgroup_timeline_us']['last_to_end']}")
             del clocks
@@ -650,9 +646,6 @@ def main():
                     help="only the projection + store measurement (with --calibrate-copy: preceded by the copy kernels "
                          "of known traffic, for a counter run)")
     ap.add_argument("--no-peaks", action="store_true", help="skip the measured GEMM / copy rates of this box")
-    ap.add_argument("--two-pass", action="store_true",
-                    help="merge split-context parts with the second kernel even where the main kernel would do it "
-                         "itself (WE_SPLIT_TWO_PASS; for same-box comparisons)")
     ap.add_argument("--two-calls", action="store_true",
                     help="we_rope_kv_store + we_attn_ring_fwd instead of the one-call we_rope_kv_attn_fwd")
     ap.add_argument("--attn-iters", type=int, default=200, help="attention-only launches for the roofline timing")

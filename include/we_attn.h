@@ -10,9 +10,9 @@
  *
  * world_engine has no native code: these are the calls a binding would replace with the
  * entry points below.  All pointers are DEVICE pointers owned by the caller.  Every call only
- * enqueues work on `stream`; it never allocates and - after the one-time set-up of the device it
- * runs on, see we_init - never synchronises, so it is re-entrant and capturable into a HIP graph.
- * The only state the library keeps is what that set-up found out about each device (read-only
+ * enqueues work on `stream`; it never allocates and never synchronises, so it is re-entrant and
+ * capturable into a HIP graph once the device it runs on has had its one-time set-up (we_init).
+ * The only state the library keeps is what that set-up noted about each device (read-only
  * afterwards).  The frame index that
  * selects the ring slot is read by the kernels from device memory (`t_pos[0]`), exactly as the
  * reference derives it from a device tensor (src/model/kv_cache.py:126), so no host value of
@@ -50,13 +50,6 @@ extern "C" {
 /* size of the library's own split-context scratch buffer (see we_attn_ring_fwd_static) */
 #define WE_STATIC_SCRATCH_BYTES (32u << 20)
 
-/* leading bytes of a split-context workspace that hold arrival counters (see we_attn_ring_fwd) */
-#define WE_WS_COUNTER_BYTES 16384
-
-/* OR into q_tile: merge split-context parts with the second kernel even where the main kernel
- * could do it itself (same results, bit for bit; for comparisons) */
-#define WE_SPLIT_TWO_PASS 0x10000
-
 /* Library version: major*10000 + minor*100 + patch. */
 int we_version(void);
 
@@ -65,13 +58,12 @@ const char* we_error_string(int code);
 
 /*
  * One-time set-up of the CURRENT device (hipSetDevice), without a counterpart in the reference:
- * raises the kernels' dynamic-LDS limits, looks up the static scratch buffer's address and runs a
- * small probe launch on the null stream that checks how the hardware deals workgroups to the
- * XCDs (the in-kernel merge of split-context parts is only used where workgroup id % 8 names the
- * XCD).  Synchronises the device once; idempotent and thread-safe.  Every entry point that
- * launches does the same implicitly on its first call on a device - except when its stream is
- * being captured, where it returns WE_ERR_NOT_READY instead: callers that capture graphs call
- * we_init() (or make one ordinary call) on the device first.
+ * raises the kernels' dynamic-LDS limits, looks up the static scratch buffer's address and notes
+ * the device's compute-unit count.  Launches nothing, does not synchronise; idempotent and
+ * thread-safe.  Every entry point that launches does the same implicitly on its first call on a
+ * device - except when its stream is being captured (these runtime calls do not belong into a
+ * capture), where it returns WE_ERR_NOT_READY instead: callers that capture graphs call we_init()
+ * (or make one ordinary call) on the device first.
  */
 int we_init(void);
 
@@ -137,9 +129,8 @@ int32_t we_attn_auto_splits(int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_
 
 /*
  * Bytes of split-context workspace we_attn_ring_fwd needs for these sizes and the given n_splits /
- * q_tile arguments (0 when nothing is split; otherwise WE_WS_COUNTER_BYTES + the partial
- * results).  Depends on the compute-unit count of the current device (256 when there is none to
- * ask).  Sizing helper without a counterpart in the reference.
+ * q_tile arguments (0 when nothing is split).  Depends on the compute-unit count of the current
+ * device (256 when there is none to ask).  Sizing helper without a counterpart in the reference.
  */
 size_t we_attn_workspace_bytes(int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L,
                                int32_t n_splits, int32_t q_tile);
@@ -147,15 +138,13 @@ size_t we_attn_workspace_bytes(int32_t B, int32_t H, int32_t Hkv, int32_t T, int
 /*
  * What the library would do with an attention call of these sizes (inspection helper without a
  * counterpart in the reference; launches nothing): plan[0] = queries per workgroup, [1] = context
- * parts of the units that are split, [2] = leading (batch, kv head) units left whole, [3] = 1 when
- * the main kernel merges the parts itself (0: second kernel), [4] = workgroups of the main launch,
- * [5] = compute units planned for.  compute_units = 0 asks the current device (256 without one);
- * xcd_merge: 1 / 0 = assume that the device passed / failed we_init's XCD check, -1 = use what the
- * current device's set-up found (runs it if need be, see we_init).
+ * parts of the units that are split, [2] = leading (batch, kv head) units left whole, [3] =
+ * workgroups of the main launch, [4] = compute units planned for.  compute_units = 0 asks the
+ * current device (256 without one).
  */
-#define WE_PLAN_FIELDS 6
+#define WE_PLAN_FIELDS 5
 int we_attn_plan(int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L, int32_t n_splits,
-                 int32_t q_tile, int32_t compute_units, int32_t xcd_merge, int32_t plan[WE_PLAN_FIELDS]);
+                 int32_t q_tile, int32_t compute_units, int32_t plan[WE_PLAN_FIELDS]);
 
 /*
  * Frame-block-causal attention of one frame's queries over the ring buffer.
@@ -172,26 +161,15 @@ int we_attn_plan(int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64
  *   kv, written, t_pos   as in we_rope_kv_store, after that call for the same frame.
  *   out  [B, H, T, Dh]   element strides out_strides = {batch, head, token}; Dh contiguous.
  *   workspace            device scratch of at least we_attn_workspace_bytes(...) bytes for the
- *                        same sizes, n_splits and q_tile; may be NULL when that is 0.  Its first
- *                        WE_WS_COUNTER_BYTES bytes hold arrival counters: they must be ZERO when
- *                        the buffer is first handed to the library, and every call leaves them
- *                        zero again (so a buffer is cleared once, when it is allocated, and can be
- *                        reused by calls of any sizes that follow each other on a stream; calls
- *                        that overlap in time need a workspace each).  The rest may hold anything.
+ *                        same sizes, n_splits and q_tile; may be NULL when that is 0.  Nothing in
+ *                        it has to start at any value; calls that overlap in time need a
+ *                        workspace each.
  *   n_splits             0 = choose automatically (small grids: every (batch, kv head) unit is
  *                        split so that most CUs have work; grids that leave a partial last round
  *                        of workgroups: only that round's units are split); 1 = single pass;
  *                        2..64 = split the visible context of every unit into that many parts.
- *                        The parts are merged by the main kernel itself - by whichever workgroup
- *                        of a query tile finishes last, through the L2 of the XCD that all parts
- *                        of a unit are placed on - when the device passed we_init's XCD check and
- *                        both the split and the unsplit unit counts are multiples of 8 (at most
- *                        16 parts); otherwise by a second kernel.  Both routes give the same
- *                        bits.  The first route relies on the placement we_init checked on the
- *                        null stream: a stream that restricts the CUs a kernel may use (a CU
- *                        mask) can place workgroups differently - pass WE_SPLIT_TWO_PASS there.
- *   q_tile               queries per workgroup: 0 = choose automatically, or 128 / 256;
- *                        optionally | WE_SPLIT_TWO_PASS.
+ *                        Split parts are combined by a second kernel.
+ *   q_tile               queries per workgroup: 0 = choose automatically, or 128 / 256.
  *   scale                softmax scale (> 0); the reference uses 1/sqrt(Dh).
  *
  * Requirements: dtype bf16 or f16 (MFMA kernel) or f32 (plain one-pass kernel on the vector
@@ -221,9 +199,8 @@ int we_attn_ring_fwd(const void* q, const int64_t q_strides[3],
  * hipMalloc / hipFree and calls no allocating library routine.
  * All calls on one GPU share that GPU's buffer: calls that overlap in time on one GPU (different
  * streams, or parallel branches of one graph) race on it; calls that follow each other on a
- * stream do not.  The buffer's arrival counters are zero when the image is loaded and every call
- * leaves them zero; nothing else in it has to start at any value (every partial row a call reads
- * was written by that call).
+ * stream do not.  Nothing in the buffer has to start at any value (every partial row a call reads
+ * was written by that call's first kernel).
  */
 int we_attn_ring_fwd_static(const void* q, const int64_t q_strides[3],
                             const void* kv, const uint8_t* written, const int64_t* t_pos,

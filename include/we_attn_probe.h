@@ -24,9 +24,7 @@ extern "C" {
  * same interval in ticks of the device's constant 100 MHz counter (their ratio is the shader
  * clock the kernel actually ran at; boards lower it under their power limit), [2 + s] the ticks
  * from its start to stage s as seen by its first thread: 0 slot list built, 1 first K tile in
- * LDS, 2 tile loop left, 3 wavefront pair merged, 4 (partial) results stored, and for workgroups
- * that merge context parts themselves 5 own partial rows acknowledged, 6 every wavefront's, 7
- * counted in, 8 shares known, 9 merged; [2 + 11] the shares it merged (bit mask).
+ * LDS, 2 tile loop left, 3 wavefront pair merged, 4 (partial) results stored.
  * clocks_len = number of uint64 elements available; at least WE_CLOCK_SLOTS * (workgroups of the
  * launch) or WE_ERR_WORKSPACE is returned; entries of workgroups that own no work, and of stages
  * a workgroup does not pass, stay untouched (zero them beforehand).  bf16 / f16 only.  Everything

@@ -85,16 +85,14 @@ def test_validation_codes_without_gpu():
 def test_workspace_and_split_planning():
     lib = _capi.lib()
     assert lib.we_attn_workspace_bytes(1, 16, 16, 256, 128, 4096, 1, 0) == 0
-    hdr = _capi.WE_WS_COUNTER_BYTES      # arrival counters at the start of every split-context workspace
-    assert lib.we_attn_workspace_bytes(1, 16, 16, 256, 128, 4096, 4, 0) == hdr + 4 * 16 * 256 * (128 * 2 + 16)
-    assert lib.we_attn_workspace_bytes(1, 16, 16, 256, 128, 4096, 4, _capi.WE_SPLIT_TWO_PASS) == hdr + 4 * 16 * 256 * (128 * 2 + 16)
+    assert lib.we_attn_workspace_bytes(1, 16, 16, 256, 128, 4096, 4, 0) == 4 * 16 * 256 * (128 * 2 + 16)
     # 256-token frames: every unit is split, into three quarters of the parts that would give every CU a workgroup
     s = lib.we_attn_auto_splits(1, 16, 16, 256, 128, 4096)
     assert s == 6
     # ... and the workgroups of a call never outnumber the 256 CUs: 48, 80, 96, 160 unsplit workgroups
     for heads, want in ((24, 5), (40, 3), (48, 2), (80, 1)):
         assert lib.we_attn_auto_splits(1, heads, heads, 256, 128, 4096) == want, heads
-    assert lib.we_attn_workspace_bytes(1, 16, 16, 256, 128, 4096, 0, 0) == hdr + s * 16 * 256 * (128 * 2 + 16)
+    assert lib.we_attn_workspace_bytes(1, 16, 16, 256, 128, 4096, 0, 0) == s * 16 * 256 * (128 * 2 + 16)
     # long contexts (32 slots and more) take about 240 workgroups; 32 heads are cut in four (all 256 CUs);
     # beyond sixteen parts about 160 workgroups
     assert lib.we_attn_auto_splits(1, 16, 16, 256, 128, 8192) == 7
@@ -105,26 +103,12 @@ def test_workspace_and_split_planning():
     # 1024-token frames with 96 heads: 384 workgroups of 256 queries = 1.5 rounds of 256 CUs, so only
     # the last 32 of the 96 units (128 workgroups) are split in two
     assert lib.we_attn_auto_splits(4, 24, 24, 1024, 128, 8192) == 2
-    assert lib.we_attn_workspace_bytes(4, 24, 24, 1024, 128, 8192, 0, 0) == hdr + 2 * 32 * 1024 * (128 * 2 + 16)
+    assert lib.we_attn_workspace_bytes(4, 24, 24, 1024, 128, 8192, 0, 0) == 2 * 32 * 1024 * (128 * 2 + 16)
     # whole rounds: nothing to split
     assert lib.we_attn_auto_splits(4, 32, 32, 1024, 128, 8192) == 1
     assert lib.we_attn_workspace_bytes(4, 32, 32, 1024, 128, 8192, 0, 0) == 0
     # never more splits than half the 64-key tiles of the context
     assert lib.we_attn_auto_splits(1, 1, 1, 64, 64, 128) <= 1
-
-
-def test_plan_reports_the_in_kernel_merge():
-    """16 units of a 256-token frame (benchmark configurations 1, 2 and 4) and the 32 tail units of
-    configuration 3 are merged in the kernel; unit counts that are not multiples of 8, a device
-    that did not pass the XCD check and the two-pass flag take the second kernel."""
-    assert ops.attn_plan(1, 16, 16, 256, 128, 4096, compute_units=256) == {
-        "q_tile": 128, "n_splits": 6, "units_whole": 0, "merge_in_kernel": True, "workgroups": 192, "compute_units": 256}
-    assert ops.attn_plan(1, 16, 16, 256, 128, 8192, compute_units=256)["merge_in_kernel"]
-    p3 = ops.attn_plan(4, 24, 24, 1024, 128, 8192, compute_units=256)
-    assert (p3["q_tile"], p3["n_splits"], p3["units_whole"], p3["merge_in_kernel"], p3["workgroups"]) == (256, 2, 64, True, 512)
-    assert not ops.attn_plan(1, 12, 12, 256, 128, 4096, compute_units=256)["merge_in_kernel"]
-    assert not ops.attn_plan(1, 16, 16, 256, 128, 4096, compute_units=256, xcd_merge=False)["merge_in_kernel"]
-    assert not ops.attn_plan(1, 16, 16, 256, 128, 4096, compute_units=256, two_pass=True)["merge_in_kernel"]
 
 
 def test_planner_over_other_shapes_and_cu_counts():
@@ -145,11 +129,13 @@ def test_planner_over_other_shapes_and_cu_counts():
                 assert pl["workgroups"] * 2 > cus or pl["n_splits"] == max(1, tiles // 2), "split calls use most of the chip"
             if unsplit >= cus and unsplit % cus == 0:
                 assert pl["n_splits"] == 1
-            if pl["merge_in_kernel"]:
-                assert pl["units_whole"] % 8 == 0 and (B * Hkv - pl["units_whole"]) % 8 == 0
     # the benchmark's 16-head call on half and on twice the CUs
     assert ops.attn_plan(1, 16, 16, 256, 128, 4096, compute_units=128)["n_splits"] == 4
     assert ops.attn_plan(1, 16, 16, 256, 128, 4096, compute_units=512)["n_splits"] == 12
+    assert ops.attn_plan(1, 16, 16, 256, 128, 4096, compute_units=256) == {
+        "q_tile": 128, "n_splits": 6, "units_whole": 0, "workgroups": 192, "compute_units": 256}
+    p3 = ops.attn_plan(4, 24, 24, 1024, 128, 8192, compute_units=256)
+    assert (p3["q_tile"], p3["n_splits"], p3["units_whole"], p3["workgroups"]) == (256, 2, 64, 512)
     # the partial last round: 384 workgroups on 256 CUs split their last 128; on 128 CUs they are three whole rounds
     assert ops.attn_plan(4, 24, 24, 1024, 128, 8192, compute_units=128)["n_splits"] == 1
 
@@ -447,7 +433,7 @@ int main(void) {
     lib = _capi.lib()
     assert int(version) == lib.we_version()
     assert int(rc_null) == -1                                    # WE_ERR_NULL_POINTER
-    assert int(ws) == _capi.WE_WS_COUNTER_BYTES + 4 * 16 * 256 * (128 * 2 + 16)
+    assert int(ws) == 4 * 16 * 256 * (128 * 2 + 16)
     assert "workspace" in msg
 
 

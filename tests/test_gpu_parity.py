@@ -239,7 +239,7 @@ def test_attention_partial_round_tail_split(gpu_device):
     assert ops.attn_auto_splits(1, 160, 160, 256, 64, 512) == 1
     assert ops.attn_workspace_bytes(1, 160, 160, 256, 64, 512) == 0
     assert ops.attn_auto_splits(1, 320, 320, 256, 64, 512) == 2
-    assert ops.attn_workspace_bytes(1, 320, 320, 256, 64, 512) == _capi.WE_WS_COUNTER_BYTES + 2 * 64 * 256 * (64 * 2 + 16)
+    assert ops.attn_workspace_bytes(1, 320, 320, 256, 64, 512) == 2 * 64 * 256 * (64 * 2 + 16)
     p = Pair(gpu_device, torch.bfloat16, B=1, H=320, Hkv=320, T=256, Dh=64, n_slots=2, cfg_id=27)
     _run_and_check(p, 4)
     p = Pair(gpu_device, torch.bfloat16, B=1, H=160, Hkv=160, T=256, Dh=64, n_slots=2, cfg_id=27)
@@ -523,7 +523,7 @@ def test_hip_graph_replay_matches_eager(gpu_device):
     layer = p.hip.layers[0]
     out_s = torch.empty(1, 4, 128, 128, dtype=torch.bfloat16, device=dev)
     n_splits = 2
-    ws = ops.new_workspace(ops.attn_workspace_bytes(1, 4, 4, 128, 128, layer.L, n_splits), dev)
+    ws = torch.empty(ops.attn_workspace_bytes(1, 4, 4, 128, 128, layer.L, n_splits), dtype=torch.uint8, device=dev)
 
     def step():
         q_rot = ops.rope_kv_store(qs, ks, vs, pos_s, p.rope.cos, p.rope.sin, p.Hgrid, p.W, layer.kv,

@@ -18,9 +18,7 @@ PROBE_LIB_PATH = os.path.join(_HERE, "libwe_probe.so")
 WE_DTYPE_BF16, WE_DTYPE_F16, WE_DTYPE_F32 = 0, 1, 2
 WE_MAX_SLOTS = 256
 WE_STATIC_SCRATCH_BYTES = 32 << 20
-WE_WS_COUNTER_BYTES = 16384
-WE_SPLIT_TWO_PASS = 0x10000
-WE_PLAN_FIELDS = 6
+WE_PLAN_FIELDS = 5
 WE_CLOCK_SLOTS = 16
 WE_ERR_SCRATCH_LIMIT = -7
 WE_ERR_NOT_READY = -8
@@ -65,7 +63,7 @@ SIGNATURES = {
     ]),
     "we_init": (c_int32, []),
     "we_attn_auto_splits": (c_int32, [c_int32, c_int32, c_int32, c_int32, c_int32, c_int64]),
-    "we_attn_plan": (c_int32, [c_int32, c_int32, c_int32, c_int32, c_int32, c_int64, c_int32, c_int32, c_int32, c_int32,
+    "we_attn_plan": (c_int32, [c_int32, c_int32, c_int32, c_int32, c_int32, c_int64, c_int32, c_int32, c_int32,
                                POINTER(c_int32)]),
     "we_attn_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32, c_int32, c_int64, c_int32, c_int32]),
     "we_attn_ring_fwd": (c_int32, [

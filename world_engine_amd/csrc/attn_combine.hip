@@ -7,8 +7,7 @@
 
 namespace we {
 
-// Second pass of the split-context path, for calls whose parts the main kernel does not merge
-// itself.  One thread per (row, 8 columns);
+// Second pass of the split-context path.  One thread per (row, 8 columns);
 // grid = (256-thread slices of one head's T * DH/8 items, split (batch, head) pairs), so that the
 // start-up code has one 32-bit division in it (the kernel is short enough for that to show).
 template <typename M, int DH>
@@ -20,7 +19,7 @@ __global__ void __launch_bounds__(256) attn_combine_kernel(AttnParams p) {
   const int64_t row = (int64_t)blockIdx.y * p.T + t;  // workspace row; query row = row + ws_row0
   const unsigned bh = (unsigned)(p.units_whole * p.group) + blockIdx.y;  // first split pair + y
   const int b = (int)(bh / (unsigned)p.H), h = (int)(bh % (unsigned)p.H);
-  merge_item<M, false, int64_t>(p, row * 16, (row * DH + dg * 8) * 2, rows * 16, rows * DH * 2, b, h, t, dg);
+  merge_item<M>(p, row * 16, (row * DH + dg * 8) * 2, rows * 16, rows * DH * 2, b, h, t, dg);
 }
 
 hipError_t launch_attn_combine(const AttnParams& p, int Dh, int dtype, hipStream_t stream) {

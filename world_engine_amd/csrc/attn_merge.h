@@ -1,28 +1,11 @@
 // Merge of split-context partial results (gfx950): one output item = 8 consecutive head-dim
-// columns of one query row.  The same function serves the second-pass kernel (attn_combine.hip)
-// and the main kernel's own merge by the last workgroup to arrive (attn_ring.hip), so that both
-// routes produce identical bits.
+// columns of one query row.  Used by the second-pass kernel (attn_combine.hip).
 #pragma once
 #include "attn_mma.h"
 #include "we_kernels.h"
 
 
 namespace we {
-
-// 16-byte load of partial results at base + lane_off + uniform_off.  L2: the load must not be
-// served from this CU's vector L1 (the partials were written by other CUs of the same XCD a moment
-// ago and live in its L2); its offsets are 32-bit (the host keeps the workspace of a call that
-// merges this way below 4 GiB) and the uniform part travels in a scalar register.
-template <bool L2, typename Off>
-__device__ __forceinline__ u32x4_t load_partial16(const void* base, Off lane_off, Off uniform_off) {
-  if constexpr (L2) {
-    const __amdgpu_buffer_rsrc_t rs =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)0xffffffffu, 0x00020000);
-    return __builtin_amdgcn_raw_buffer_load_b128(rs, (int)lane_off, (int)uniform_off, 16 /* sc1: miss the vector L1 */);
-  } else {
-    return *reinterpret_cast<const u32x4_t*>(static_cast<const unsigned char*>(base) + lane_off + uniform_off);
-  }
-}
 
 // Every split left, per query row, its normalised output as fp16 values times a row scale r_s, its
 // reference m_s (log2 domain) and its sum l_s; the result is sum_s w_s r_s O_s / sum_s w_s with
@@ -36,24 +19,21 @@ struct PartialBatch {
 
 // Requests splits [s0, s0 + 8) of one item: ml_off / o_off are the byte offsets of split 0's record
 // and of its 8 columns in the two workspace areas, ml_step / o_step the distance between splits.
-// Off is uint32_t for the in-kernel merge and int64_t for the second-pass kernel.  (The in-kernel
-// merge runs once per launch, straight out of memory and on one wavefront's issue rate: every
-// instruction of address arithmetic saved here is time off the end of the kernel.)
-template <bool L2, typename Off>
-__device__ __forceinline__ void load_batch(PartialBatch& pb, const AttnParams& p, Off ml_off, Off o_off, Off ml_step,
-                                           Off o_step, int s0) {
-  Off ml_s = (Off)s0 * ml_step, o_s = (Off)s0 * o_step;   // uniform
+__device__ __forceinline__ void load_batch(PartialBatch& pb, const AttnParams& p, int64_t ml_off, int64_t o_off,
+                                           int64_t ml_step, int64_t o_step, int s0) {
+  const unsigned char* ml = reinterpret_cast<const unsigned char*>(p.ws_ml) + ml_off + (int64_t)s0 * ml_step;
+  const unsigned char* ov = reinterpret_cast<const unsigned char*>(p.ws_o) + o_off + (int64_t)s0 * o_step;
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     if (s0 + j < p.n_splits) {  // (uniform: a request is 16 cycles of the CU's address path whether wanted or not)
-      pb.ml[j] = __builtin_bit_cast(f32x4_t, load_partial16<L2, Off>(p.ws_ml, ml_off, ml_s));
-      pb.ov[j] = __builtin_bit_cast(f16x8_t, load_partial16<L2, Off>(p.ws_o, o_off, o_s));
+      pb.ml[j] = *reinterpret_cast<const f32x4_t*>(ml);
+      pb.ov[j] = *reinterpret_cast<const f16x8_t*>(ov);
     } else {
       pb.ml[j] = f32x4_t{-INFINITY, 0.f, 0.f, 0.f};
       pb.ov[j] = f16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
     }
-    ml_s += ml_step;
-    o_s += o_step;
+    ml += ml_step;
+    ov += o_step;
   }
 }
 
@@ -98,9 +78,9 @@ __device__ __forceinline__ void finish_item(const AttnParams& p, const float (&a
 
 // One output item, any number of splits: ml_off / o_off / ml_step / o_step as for load_batch, query
 // row (b, h, t), columns [8 dg, 8 dg + 8).
-template <typename M, bool L2, typename Off>
-__device__ __forceinline__ void merge_item(const AttnParams& p, Off ml_off, Off o_off, Off ml_step, Off o_step, int b,
-                                           int h, int t, int dg) {
+template <typename M>
+__device__ __forceinline__ void merge_item(const AttnParams& p, int64_t ml_off, int64_t o_off, int64_t ml_step,
+                                           int64_t o_step, int b, int h, int t, int dg) {
   float mmax = -INFINITY, den = 0.f;
   float acc[8];
 #pragma unroll
@@ -108,7 +88,7 @@ __device__ __forceinline__ void merge_item(const AttnParams& p, Off ml_off, Off 
 #pragma nounroll
   for (int s0 = 0; s0 < p.n_splits; s0 += 8) {
     PartialBatch pb;
-    load_batch<L2, Off>(pb, p, ml_off, o_off, ml_step, o_step, s0);
+    load_batch(pb, p, ml_off, o_off, ml_step, o_step, s0);
     accumulate_batch(pb, p.n_splits - s0, mmax, den, acc);
   }
   finish_item<M>(p, acc, den, b, h, t, dg);

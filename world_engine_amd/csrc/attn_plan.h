@@ -24,19 +24,12 @@ inline int ring_shape_ok(int B, int H, int Hkv, int T, int Dh, int64_t L, int di
   return WE_OK;
 }
 
-// Arrival counters of the in-kernel merge: one region per XCD (regions never share a cache line,
-// the L2s of different XCDs are not coherent with each other inside a kernel), kCtrPerXcd counters
-// each, at the start of the workspace.
-constexpr int kCtrPerXcd = WE_WS_COUNTER_BYTES / 8 / 4;
-
 struct AttnPlan {
   int variant;      // 1: 128 queries per workgroup, 2: 256
   int block_m;      // queries per workgroup
   int n_splits;     // context splits of the units that are split (1: none)
   int units_whole;  // leading (batch, kv head) units that are not split
   int64_t ws_rows;  // query rows that go through the split-context workspace
-  int merge;        // 1: the main kernel merges the parts itself (no second launch)
-  int merge_wait;   // merge: 100 MHz ticks a part waits for the others before giving up its share
 };
 
 inline int variant_of(int q_tile) {
@@ -58,12 +51,7 @@ inline int variant_of(int q_tile) {
 //    than two 64-key tiles per part.
 //  * Many workgroups that do not divide into whole rounds of CUs (e.g. 384 on 256): only the units
 //    of the last, partial round are split, so that round finishes in a fraction of the time.
-//  * The parts of a unit are merged by the main kernel itself (shared out among a query tile's
-//    workgroups once the last of them is done) when `allow_merge`, there are at most 16 parts and
-//    all of a unit's workgroups can be placed on one XCD with the XCDs evenly loaded; otherwise by
-//    the second kernel.
-inline AttnPlan plan_attn(int B, int H, int Hkv, int T, int64_t L, int n_splits, int variant, int cus,
-                          bool allow_merge) {
+inline AttnPlan plan_attn(int B, int H, int Hkv, int T, int64_t L, int n_splits, int variant, int cus) {
   AttnPlan pl;
   if (cus < 8) cus = 8;
   const int64_t wg256 = (int64_t)B * H * ((T + 255) / 256);
@@ -120,29 +108,20 @@ inline AttnPlan plan_attn(int B, int H, int Hkv, int T, int64_t L, int n_splits,
   }
   const int split_units = units - pl.units_whole;
   pl.ws_rows = pl.n_splits > 1 ? (int64_t)split_units * group * T : 0;
-  // In-kernel merge: whole units per XCD (8 XCDs or a divisor of 8), XCDs evenly loaded, the
-  // arrival counters of an XCD within its region.
-  pl.merge = allow_merge && pl.n_splits > 1 && pl.n_splits <= 16 && pl.units_whole % 8 == 0 && split_units % 8 == 0 &&
-             (int64_t)(split_units / 8) * members <= kCtrPerXcd;
-  // Waiting for the other parts is only sound when they are certain to be running: the split
-  // units come last in the launch, so that holds when their workgroups fit the CUs together.
-  // 20 us: an order of magnitude above the spread of the parts' finishing times.
-  pl.merge_wait = pl.merge && (int64_t)split_units * members * pl.n_splits <= cus ? 2000 : 0;
   return pl;
 }
 
 inline size_t workspace_bytes_of(const AttnPlan& pl, int Dh) {
   if (pl.n_splits <= 1 || pl.ws_rows <= 0) return 0;
-  return (size_t)WE_WS_COUNTER_BYTES + (size_t)pl.n_splits * (size_t)pl.ws_rows * ((size_t)Dh * 2 + 4 * sizeof(float));
+  return (size_t)pl.n_splits * (size_t)pl.ws_rows * ((size_t)Dh * 2 + 4 * sizeof(float));
 }
 
-// Validation of a we_attn_ring_fwd call, its plan and its kernel parameters.  `q_tile` may carry
-// WE_SPLIT_TWO_PASS; `cus` and `xcd_merge_ok` describe the device the call will run on.
+// Validation of a we_attn_ring_fwd call, its plan and its kernel parameters.  `cus`: compute units
+// of the device the call will run on.
 inline int prepare_attn(const void* q, const int64_t* q_strides, const void* kv, const uint8_t* written,
                         const int64_t* t_pos, void* out, const int64_t* out_strides, void* workspace,
                         size_t workspace_bytes, int B, int H, int Hkv, int T, int Dh, int64_t L, int dilation,
-                        float scale, int n_splits, int q_tile, int dtype, int cus, bool xcd_merge_ok, AttnParams& p,
-                        AttnPlan& pl) {
+                        float scale, int n_splits, int q_tile, int dtype, int cus, AttnParams& p, AttnPlan& pl) {
   if (!q || !q_strides || !kv || !written || !t_pos || !out || !out_strides) return WE_ERR_NULL_POINTER;
   int rc = ring_shape_ok(B, H, Hkv, T, Dh, L, dilation);
   if (rc != WE_OK) return rc;
@@ -151,8 +130,6 @@ inline int prepare_attn(const void* q, const int64_t* q_strides, const void* kv,
   if (L / T > WE_MAX_SLOTS) return WE_ERR_UNSUPPORTED;
   if ((uint64_t)(L + T) * (uint64_t)Dh * 2u >= (1ull << 32)) return WE_ERR_UNSUPPORTED;  // 32-bit tile offsets
   if (!(scale > 0.f) || n_splits < 0 || n_splits > 64) return WE_ERR_BAD_SHAPE;
-  const bool two_pass = (q_tile & WE_SPLIT_TWO_PASS) != 0;
-  q_tile &= ~WE_SPLIT_TWO_PASS;
   if (variant_of(q_tile) < 0) return WE_ERR_UNSUPPORTED;
   if (dtype == WE_DTYPE_F32) {
     // fp32 caches take the plain one-pass kernel: no context splitting, no tile choice
@@ -163,17 +140,15 @@ inline int prepare_attn(const void* q, const int64_t* q_strides, const void* kv,
       !strides_ok(out_strides, dtype))
     return WE_ERR_ALIGNMENT;
 
-  pl = plan_attn(B, H, Hkv, T, L, n_splits, variant_of(q_tile), cus, xcd_merge_ok && !two_pass);
+  pl = plan_attn(B, H, Hkv, T, L, n_splits, variant_of(q_tile), cus);
   const size_t ws_need = workspace_bytes_of(pl, Dh);
-  if (ws_need >= (1ull << 32)) pl.merge = 0;  // the merge addresses the workspace with 32-bit offsets
   if (ws_need > 0) {
     if (!workspace || !aligned16(workspace)) return WE_ERR_WORKSPACE;
     if (workspace_bytes < ws_need) return WE_ERR_WORKSPACE;
   }
 
   p.q = q; p.kv = kv; p.written = written; p.t_pos = t_pos; p.out = out;
-  p.ws_ctr = ws_need ? static_cast<uint32_t*>(workspace) : nullptr;
-  p.ws_o = ws_need ? reinterpret_cast<uint16_t*>(static_cast<unsigned char*>(workspace) + WE_WS_COUNTER_BYTES) : nullptr;
+  p.ws_o = ws_need ? static_cast<uint16_t*>(workspace) : nullptr;
   p.ws_ml = ws_need ? reinterpret_cast<float*>(p.ws_o + (size_t)pl.n_splits * (size_t)pl.ws_rows * Dh) : nullptr;
   p.qs_b = q_strides[0]; p.qs_h = q_strides[1]; p.qs_t = q_strides[2];
   p.os_b = out_strides[0]; p.os_h = out_strides[1]; p.os_t = out_strides[2];
@@ -187,12 +162,6 @@ inline int prepare_attn(const void* q, const int64_t* q_strides, const void* kv,
   p.group = H / Hkv;
   p.members = p.group * p.q_tiles;
   p.unit_splits = pl.units_whole + (B * Hkv - pl.units_whole) * pl.n_splits;
-  if ((int64_t)B * H * T >= (1ll << 31)) pl.merge = 0;  // ... and rows with 32-bit indices
-  p.merge = pl.merge;
-  p.merge_wait = pl.merge ? pl.merge_wait : 0;
-  p.ws_rows32 = (uint32_t)pl.ws_rows;
-  p.ws_row0_32 = (uint32_t)p.ws_row0;
-  p.share_items = (uint32_t)((pl.block_m * (Dh / 8) + pl.n_splits - 1) / pl.n_splits);
   p.scale_log2 = scale * 1.4426950408889634f;
   p.gate = nullptr; p.gs_b = p.gs_h = p.gs_t = 0;
   p.gate_x = nullptr; p.gate_w = nullptr; p.gx_b = p.gx_t = 0;
@@ -212,7 +181,7 @@ inline int launch_attn(const AttnParams& p, const AttnPlan& pl, int Dh, int dtyp
   if (dtype == WE_DTYPE_BF16) e = Dh == 128 ? launch_attn_ring_bf16_128(p, ksplit, st) : launch_attn_ring_bf16_64(p, ksplit, st);
   else e = Dh == 128 ? launch_attn_ring_f16_128(p, ksplit, st) : launch_attn_ring_f16_64(p, ksplit, st);
   if (e != hipSuccess) return WE_ERR_LAUNCH;
-  if (pl.n_splits > 1 && !pl.merge && launch_attn_combine(p, Dh, dtype, st) != hipSuccess) return WE_ERR_LAUNCH;
+  if (pl.n_splits > 1 && launch_attn_combine(p, Dh, dtype, st) != hipSuccess) return WE_ERR_LAUNCH;
   return WE_OK;
 }
 

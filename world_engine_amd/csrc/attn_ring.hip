@@ -32,10 +32,7 @@
 // reads ahead of their MFMAs, also across steps and barriers, and the order is pinned with
 // sched_barrier.  When the workgroup count leaves a partial last round of CUs, only that round's
 // (batch, kv head) units are context-split (see the planner in attn_plan.h); split workgroups leave
-// normalised partial outputs.  Those are merged either by a second kernel (attn_combine.hip), or -
-// when the planner could place all workgroups of a unit on one XCD - by this kernel itself: the
-// parts of a query tile count their arrivals and whichever finishes last merges them, reading the
-// others' rows out of the XCD's L2 (no second launch, no trip of the partials through HBM).
+// normalised partial outputs that a second kernel merges (attn_combine.hip).
 //
 // The grid is 3-D (8 * query tiles, query heads per kv head, rounds of 8 units): no division by
 // run-time values is needed to find a workgroup's unit, and blockIdx.x % 8 is the XCD it runs on,
@@ -46,9 +43,10 @@
 // of a slot is loaded with its missing rows clamped and its missing keys masked to -inf.
 //
 // Roofline: 4*T*N_vis*Dh flops and 4*N_vis*Dh bytes of K/V per (batch, kv head).
-#include "attn_merge.h"
-#include "attn_plan.h"
+#include "attn_mma.h"
 #include "device_state.h"
+#include "we_kernels.h"
+#include "../../include/we_attn.h"
 
 #include <type_traits>
 
@@ -143,30 +141,17 @@ attn_ring_kernel(AttnParams p) {
   // to XCDs round-robin in linear order, so XCD = blockIdx.x % 8, and the workgroups that share
   // one K/V stream (the x * y of one round) all land on the same XCD and its L2.
   const int xcd = blockIdx.x & 7, qtile = blockIdx.x >> 3, hq_in = blockIdx.y;
+  const int us_raw = blockIdx.z * 8 + xcd;
+  // a workgroup past the end computes the addresses of the last one and leaves further down, so
+  // that the requests above and below do not wait behind a branch
+  const int us = us_raw < p.unit_splits ? us_raw : p.unit_splits - 1;
   // leading units run unsplit; the rest are cut into n_splits context parts each
-  int unit, split, nsp, us_raw;
-  if (p.merge) {
-    // all parts of a unit on this XCD (the planner made both unit counts multiples of 8): rounds
-    // [0, units_whole / 8) hold the whole units, then every eight split units take n_splits rounds
-    const int zw = p.units_whole >> 3;
-    us_raw = 0;  // (the grid has no workgroup past the end)
-    if ((int)blockIdx.z < zw) {
-      unit = blockIdx.z * 8 + xcd; split = 0; nsp = 1;
-    } else {
-      const int zz = blockIdx.z - zw;
-      unit = p.units_whole + (zz / p.n_splits) * 8 + xcd; split = zz % p.n_splits; nsp = p.n_splits;
-    }
+  int unit, split, nsp;
+  if (us < p.units_whole) {
+    unit = us; split = 0; nsp = 1;
   } else {
-    us_raw = blockIdx.z * 8 + xcd;
-    // a workgroup past the end computes the addresses of the last one and leaves further down, so
-    // that the requests above and below do not wait behind a branch
-    const int us = us_raw < p.unit_splits ? us_raw : p.unit_splits - 1;
-    if (us < p.units_whole) {
-      unit = us; split = 0; nsp = 1;
-    } else {
-      const int r = us - p.units_whole;
-      unit = p.units_whole + r / p.n_splits; split = r % p.n_splits; nsp = p.n_splits;
-    }
+    const int r = us - p.units_whole;
+    unit = p.units_whole + r / p.n_splits; split = r % p.n_splits; nsp = p.n_splits;
   }
   const int b = unit / p.Hkv, hkv = unit - b * p.Hkv;
   const int h = hkv * p.group + hq_in;
@@ -695,8 +680,6 @@ attn_ring_kernel(AttnParams p) {
   half_wave_pair(l_run, lo, up);
   float l_tot = lo + up;
   m_ref *= lmul;  // from raw logits to the log2 domain the merges work in
-  // this kernel merges the context parts itself: every wavefront stays to the end
-  const bool merging = p.merge != 0 && nsp > 1;
 
   if (KSPLIT == 2) {
     // ---- the two wavefronts of a query block merge their (m, l, O) through LDS ----
@@ -712,8 +695,7 @@ attn_ring_kernel(AttnParams p) {
       mb[(DB * 4) * 64] = f32x4_t{m_ref, l_tot, 0.f, 0.f};
     }
     __syncthreads();
-    if (hb == 1 && !merging) return;
-    if (hb == 0) {
+    if (hb == 1) return;
     const f32x4_t ml1 = mb[(DB * 4) * 64];
     // a wavefront whose sum is zero saw no key (or only keys that vanish against its reference):
     // its reference must not take part in the maximum
@@ -733,12 +715,10 @@ attn_ring_kernel(AttnParams p) {
       l_tot = a0 * l_tot + a1 * l1;
       m_ref = mm;
     }
-    }
   }
 
   stamp(3);  // pair merged
   // ---- epilogue ----
-  if (KSPLIT == 1 || hb == 0) {
   const int64_t rows = (int64_t)p.B * p.H * p.T - p.ws_row0;  // rows in the workspace
   const bool valid = qrow < p.T;
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
@@ -806,95 +786,7 @@ attn_ring_kernel(AttnParams p) {
       }
     }
   }
-  }  // (epilogue of the wavefronts that hold results)
   stamp(4);  // results / partial results stored (requests issued)
-
-  // ---- merge of the context parts, shared out among the workgroups that computed them ----
-  // Every part has left its rows in the workspace with plain stores, i.e. in the L2 of the XCD that
-  // all parts of a unit run on.  Once a workgroup's own rows are there (its wavefronts' store
-  // counters at zero, then the barrier) it counts itself in on the tile's arrival word.  The merge
-  // of the tile's BM x Dh outputs is cut into one share per part: the workgroup that finds all
-  // others counted merges its own share at once; the others look at the word for a bounded time
-  // (the parts of a tile finish within a microsecond or two of each other) and merge their share
-  // when the count is complete, so that the merge costs every CU a share of the reads instead of
-  // one CU all of them.  A workgroup that will not wait (any longer) says so in the word and goes;
-  // the last to arrive takes the shares of those that left.  All of this goes through one word per
-  // tile, whose atomic operations are ordered, so every share is merged exactly once, after every
-  // part is in, and nobody waits without a limit.  Partial rows are read with loads that miss the
-  // CU's own L1; the arithmetic is the second-pass kernel's.  The word is zero again once every
-  // workgroup has stopped looking at it, which is how the next call expects to find it.
-  //   word: bits 7:0 parts arrived, 15:8 parts departed, 31:16 shares given up by their owners
-  if (merging) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    stamp(5);  // this wavefront's partial rows acknowledged
-    __syncthreads();
-    stamp(6);  // every wavefront's
-    volatile uint32_t* todo = reinterpret_cast<volatile uint32_t*>(smem + L::MISC_OFF);
-    uint32_t* word = p.ws_ctr + xcd * host::kCtrPerXcd +
-                     ((((unit - p.units_whole) >> 3) * p.group + hq_in) * p.q_tiles + qtile);
-    const uint32_t parts = (uint32_t)nsp;
-    uint32_t departed = 0;
-    if (tid == 0) {
-      uint32_t mine = 0;
-      const uint32_t before = __hip_atomic_fetch_add(word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-      if (CLOCKED) asm volatile("" ::"v"(before));
-      stamp(7);  // counted in
-      if ((before & 0xffu) + 1u == parts) {
-        mine = (before >> 16) | (1u << split);  // last in: its own share and those given up
-      } else {
-        bool all_in = false;
-        if (p.merge_wait > 0) {
-          const uint64_t t0 = __builtin_amdgcn_s_memrealtime();  // constant 100 MHz counter
-          do {
-            __builtin_amdgcn_s_sleep(4);
-            all_in = (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & 0xffu) == parts;
-          } while (!all_in && __builtin_amdgcn_s_memrealtime() - t0 < (uint64_t)p.merge_wait);
-        }
-        if (!all_in) {
-          // giving up the share - unless everyone was in before the mark, in which case the last
-          // one in has not seen it and the share is still this workgroup's
-          const uint32_t seen = __hip_atomic_fetch_or(word, 1u << (16 + split), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-          all_in = (seen & 0xffu) == parts;
-        }
-        if (all_in) mine = 1u << split;
-      }
-      *todo = mine;
-      // This workgroup will not look at the word again: it departs now, so that the operation's
-      // round trip runs under the merge below.  The last to depart puts the word back to zero.
-      departed = __hip_atomic_fetch_add(word, 0x100u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    }
-    // (a bare barrier after the LDS write has landed: __syncthreads() would first wait for the
-    // departure's answer, which nobody needs before the end)
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    const uint32_t shares = (uint32_t)__builtin_amdgcn_readfirstlane((int)*todo);
-    stamp(8);  // shares known: every part is in (or this workgroup has given up)
-    if (CLOCKED && tid == 0) p.clock_out[kClockSlots * wg_id + 2 + 11] = shares;
-    // (row, 8 columns) items: 16 (Dh 128) or 8 consecutive lanes share a row, so requests cover
-    // whole rows.  Nothing is unrolled and all offsets are 32-bit (the host saw to it that they
-    // fit): this code runs once per launch, at one instruction per few cycles.  From four parts on
-    // a share is one item per thread.
-    constexpr uint32_t DG = DH / 8, N = BM * DG;
-    const int t0 = qtile * BM;
-    const uint32_t wrow0 = (uint32_t)((b * p.H + h) * p.T + t0) - p.ws_row0_32;  // tile's first row in the workspace
-    const uint32_t ml_step = p.ws_rows32 * 16u, o_step = p.ws_rows32 * (uint32_t)(DH * 2);
-#pragma nounroll
-    for (uint32_t left = shares; left != 0u; left &= left - 1u) {
-      const uint32_t lo = (uint32_t)__builtin_ctz(left) * p.share_items;
-      const uint32_t hi = lo + p.share_items < N ? lo + p.share_items : N;
-#pragma nounroll
-      for (uint32_t it = lo + tid; it < hi; it += 512u) {
-        const uint32_t r = it / DG, dg = it % DG;
-        if (t0 + (int)r < p.T)
-          merge_item<M, true, uint32_t>(p, (wrow0 + r) * 16u, ((wrow0 + r) * DH + dg * 8u) * 2u, ml_step, o_step, b, h,
-                                        t0 + (int)r, (int)dg);
-      }
-    }
-    stamp(9);  // merged (requests issued)
-    if (tid == 0 && ((departed >> 8) & 0xffu) + 1u == parts)
-      __hip_atomic_store(word, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-  }
   if (CLOCKED && tid == 0) {
     p.clock_out[kClockSlots * wg_id] = (uint64_t)__builtin_readcyclecounter() - clk0;
     p.clock_out[kClockSlots * wg_id + 1] = (uint64_t)__builtin_amdgcn_s_memrealtime() - wall0;

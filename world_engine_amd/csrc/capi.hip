@@ -28,7 +28,7 @@ Dev dev_for(hipStream_t st) {
   const DeviceState* ds = nullptr;
   Dev d;
   d.rc = we::host::device_state(st, &ds);
-  d.state = ds ? *ds : DeviceState{256, false, nullptr};
+  d.state = ds ? *ds : DeviceState{256, nullptr};
   return d;
 }
 
@@ -38,7 +38,7 @@ int prepare_attn(const DeviceState& ds, const void* q, const int64_t* q_strides,
                  int B, int H, int Hkv, int T, int Dh, int64_t L, int dilation, float scale, int n_splits, int q_tile,
                  int dtype, we::AttnParams& p, AttnPlan& pl) {
   return we::host::prepare_attn(q, q_strides, kv, written, t_pos, out, out_strides, workspace, workspace_bytes, B, H,
-                                Hkv, T, Dh, L, dilation, scale, n_splits, q_tile, dtype, ds.cus, ds.xcd_merge, p, pl);
+                                Hkv, T, Dh, L, dilation, scale, n_splits, q_tile, dtype, ds.cus, p, pl);
 }
 
 // Validation of a we_rope_kv_store call and its kernel parameters.
@@ -227,43 +227,34 @@ int we_init(void) { return we::host::init_current_device(); }
 int32_t we_attn_auto_splits(int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L) {
   (void)Dh;
   if (B <= 0 || H <= 0 || Hkv <= 0 || H % Hkv != 0 || T <= 0 || L <= 0) return 1;
-  return plan_attn(B, H, Hkv, T, L, 0, 0, we::host::compute_units(), false).n_splits;
+  return plan_attn(B, H, Hkv, T, L, 0, 0, we::host::compute_units()).n_splits;
 }
 
 size_t we_attn_workspace_bytes(int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L,
                                int32_t n_splits, int32_t q_tile) {
   if (B <= 0 || H <= 0 || Hkv <= 0 || H % Hkv != 0 || T <= 0 || Dh <= 0 || L <= 0 || n_splits < 0) return 0;
-  const int variant = variant_of(q_tile & ~WE_SPLIT_TWO_PASS);
+  const int variant = variant_of(q_tile);
   if (variant < 0) return 0;
-  return workspace_bytes_of(plan_attn(B, H, Hkv, T, L, n_splits, variant, we::host::compute_units(), false), Dh);
+  return workspace_bytes_of(plan_attn(B, H, Hkv, T, L, n_splits, variant, we::host::compute_units()), Dh);
 }
 
 int we_attn_plan(int32_t B, int32_t H, int32_t Hkv, int32_t T, int32_t Dh, int64_t L, int32_t n_splits,
-                 int32_t q_tile, int32_t compute_units, int32_t xcd_merge, int32_t plan[WE_PLAN_FIELDS]) {
+                 int32_t q_tile, int32_t compute_units, int32_t plan[WE_PLAN_FIELDS]) {
   if (!plan) return WE_ERR_NULL_POINTER;
   if (B <= 0 || H <= 0 || Hkv <= 0 || H % Hkv != 0 || T <= 0 || Dh <= 0 || L <= 0 || L % T != 0 || n_splits < 0 ||
       n_splits > 64 || compute_units < 0)
     return WE_ERR_BAD_SHAPE;
-  const bool two_pass = (q_tile & WE_SPLIT_TWO_PASS) != 0;
-  const int variant = variant_of(q_tile & ~WE_SPLIT_TWO_PASS);
+  const int variant = variant_of(q_tile);
   if (variant < 0) return WE_ERR_UNSUPPORTED;
   const int cus = compute_units > 0 ? compute_units : we::host::compute_units();
-  if (xcd_merge < 0) {  // what the current device's set-up found
-    const DeviceState* ds = nullptr;
-    const int rc = we::host::device_state(nullptr, &ds);
-    if (rc != WE_OK) return rc;
-    xcd_merge = ds->xcd_merge ? 1 : 0;
-  }
-  AttnPlan pl = plan_attn(B, H, Hkv, T, L, n_splits, variant, cus, xcd_merge != 0 && !two_pass);
-  if (workspace_bytes_of(pl, Dh) >= (1ull << 32)) pl.merge = 0;
+  const AttnPlan pl = plan_attn(B, H, Hkv, T, L, n_splits, variant, cus);
   const int q_tiles = (T + pl.block_m - 1) / pl.block_m;
   const int64_t wgs = (int64_t)q_tiles * (H / Hkv) * (pl.units_whole + (int64_t)(B * Hkv - pl.units_whole) * pl.n_splits);
   plan[0] = pl.block_m;
   plan[1] = pl.n_splits;
   plan[2] = pl.units_whole;
-  plan[3] = pl.merge;
-  plan[4] = (int32_t)(wgs > 0x7fffffff ? 0x7fffffff : wgs);
-  plan[5] = cus;
+  plan[3] = (int32_t)(wgs > 0x7fffffff ? 0x7fffffff : wgs);
+  plan[4] = cus;
   return WE_OK;
 }
 

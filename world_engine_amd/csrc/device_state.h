@@ -6,23 +6,21 @@ namespace we {
 namespace host {
 
 struct DeviceState {
-  int cus;         // compute units
-  bool xcd_merge;  // workgroup id % 8 names the XCD a workgroup runs on (verified by a probe launch)
-  void* scratch;   // device address of the library's static split-context buffer on this device
+  int cus;        // compute units
+  void* scratch;  // device address of the library's static split-context buffer on this device
 };
 
 // Compute units of the current device (256 when no device can be asked, e.g. on a build host).
 // Cheap, never synchronises, safe under stream capture.
 int compute_units();
 
-// One-time set-up of the current device: kernel LDS limits, the static buffer's address, the probe
-// launch that checks the workgroup -> XCD mapping.  Synchronises the device once; later calls
-// return at once.
+// One-time set-up of the current device: kernel LDS limits, the static buffer's address, the
+// compute-unit count.  Launches nothing and does not synchronise; later calls return at once.
 int init_current_device();
 
 // State of the current device for a call that will enqueue on `stream`.  Sets the device up on
-// first use - unless `stream` is being captured, where set-up (a synchronising probe launch) is
-// not possible: WE_ERR_NOT_READY then.
+// first use - unless `stream` is being captured (the set-up's runtime calls do not belong into a
+// capture): WE_ERR_NOT_READY then.
 int device_state(hipStream_t stream, const DeviceState** out);
 
 }  // namespace host

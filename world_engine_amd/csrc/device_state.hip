@@ -12,46 +12,14 @@
 // that the entry point needs no allocation and no caller-owned workspace.  Every GPU the library
 // runs on holds its own copy at its own address; host code must never use the array's name as an
 // address (on the host it is a stand-in for the symbol), only what hipGetSymbolAddress returns
-// with the device in question current.  Zero when the image is loaded, which is what the arrival
-// counters at its start need.
+// with the device in question current.
 static __device__ __align__(256) unsigned char scratch[WE_STATIC_SCRATCH_BYTES];
-
-// XCC id of every workgroup of the probe launch.
-static __device__ uint32_t xcc_seen[1024];
 
 namespace we {
 
 namespace {
 
 constexpr int kMaxDevices = 64;
-constexpr unsigned kProbeX = 32, kProbeY = 2, kProbeZ = 3;
-
-// Every workgroup records the id of the XCD (accelerator complex) it runs on.
-__global__ void xcc_probe_kernel(uint32_t* out) {
-  const uint32_t xcc = __builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11)) & 0xfu;  // HW_REG_XCC_ID, bits 3:0
-  if (threadIdx.x == 0) out[blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z)] = xcc;
-}
-
-// The in-kernel merge of split-context partials relies on all workgroups with the same
-// blockIdx.x % 8 (grid x a multiple of 8) running on one XCD, i.e. sharing one L2.  The hardware
-// deals workgroups to the XCDs of a partition round-robin in linear order; this launch checks that
-// on the device at hand instead of assuming it.
-bool probe_xcd_mapping() {
-  void* out = nullptr;
-  if (hipGetSymbolAddress(&out, HIP_SYMBOL(xcc_seen)) != hipSuccess || out == nullptr) return false;
-  hipLaunchKernelGGL(xcc_probe_kernel, dim3(kProbeX, kProbeY, kProbeZ), dim3(64), 0, nullptr, static_cast<uint32_t*>(out));
-  if (hipGetLastError() != hipSuccess) return false;
-  uint32_t seen[kProbeX * kProbeY * kProbeZ];
-  if (hipMemcpy(seen, out, sizeof(seen), hipMemcpyDeviceToHost) != hipSuccess) return false;
-  uint32_t of_slot[8];
-  for (unsigned i = 0; i < kProbeX * kProbeY * kProbeZ; ++i) {
-    const unsigned slot = (i % kProbeX) & 7u;
-    if (i < 8) of_slot[slot] = seen[i];
-    else if (seen[i] != of_slot[slot]) return false;
-  }
-  return true;
-}
-
 struct Entry {
   std::atomic<bool> ready{false};
   host::DeviceState st{};
@@ -90,7 +58,6 @@ int init_current_device() {
   if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) return WE_ERR_LAUNCH;
   e.st.scratch = p;
   e.st.cus = compute_units();
-  e.st.xcd_merge = probe_xcd_mapping();
   e.ready.store(true, std::memory_order_release);
   return WE_OK;
 }

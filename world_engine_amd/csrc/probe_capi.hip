@@ -24,8 +24,7 @@ int we_attn_ring_fwd_clocked(const void* q, const int64_t q_strides[3], const vo
   we::AttnParams p;
   we::host::AttnPlan pl;
   const int rc = we::host::prepare_attn(q, q_strides, kv, written, t_pos, out, out_strides, workspace, workspace_bytes,
-                                        B, H, Hkv, T, Dh, L, dilation, scale, n_splits, q_tile, dtype, ds->cus,
-                                        ds->xcd_merge, p, pl);
+                                        B, H, Hkv, T, Dh, L, dilation, scale, n_splits, q_tile, dtype, ds->cus, p, pl);
   if (rc != WE_OK) return rc;
   const size_t wgs = (size_t)(8 * p.q_tiles) * (size_t)p.group * (size_t)((p.unit_splits + 7) / 8);
   if (clocks_len < WE_CLOCK_SLOTS * wgs) return WE_ERR_WORKSPACE;

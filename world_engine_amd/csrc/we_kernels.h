@@ -46,7 +46,6 @@ struct AttnParams {
   void* out;
   uint16_t* ws_o;  // [n_splits][rows >= ws_row0][Dh] normalised partial outputs / row scale, fp16 in [-1, 1]
   float* ws_ml;    // [n_splits][rows >= ws_row0][4]  softmax reference (log2 domain), sum, row scale, unused
-  uint32_t* ws_ctr;  // arrival counters of the in-kernel merge: 8 regions (one per XCD), zero between calls
   int64_t qs_b, qs_h, qs_t;
   int64_t os_b, os_h, os_t;
   int64_t L;
@@ -59,12 +58,6 @@ struct AttnParams {
   int group;        // query heads per kv head, H / Hkv
   int members;      // workgroups that share one K/V stream: group * q_tiles
   int unit_splits;  // units_whole + (B * Hkv - units_whole) * n_splits
-  int merge;        // split parts are merged by the main kernel (all workgroups of a unit on one XCD)
-  int merge_wait;   // ticks of the 100 MHz counter a part waits for the others before it gives up its share (0: none)
-  // in-kernel merge, precomputed so that the kernel's tail has no divisions and no 64-bit arithmetic:
-  uint32_t ws_rows32;    // rows of the workspace
-  uint32_t ws_row0_32;   // ws_row0
-  uint32_t share_items;  // (row, 8 columns) items of a query tile per share: ceil(queries per workgroup * Dh / 8 / n_splits)
   float scale_log2;  // softmax scale * log2(e), applied to the raw logits in fp32
   // optional per (batch, head, token) output gate, element type (src/model/attn.py:117-119): either
   // given (sigmoid applied), or computed here from the module's input and gate_proj.weight

@@ -158,7 +158,7 @@ class LayerKVCache(nn.Module):
                 ws_bytes = ops.attn_workspace_bytes(B, H, k.shape[1], T, Dh, self.L)
                 kept[key] = dict(q_rot=torch.empty((B, H, T, Dh), dtype=q.dtype, device=q.device),
                                  out=torch.empty((B, T, H, Dh), dtype=q.dtype, device=q.device).transpose(1, 2),
-                                 workspace=ops.new_workspace(ws_bytes, q.device) if ws_bytes else None)
+                                 workspace=torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None)
             bufs = kept[key]
         return ops.rope_kv_attn(q, k, v, pos_ids, rope.cos, rope.sin, rope.height, rope.width, self.kv,
                                 self.written, self.L, self.pinned_dilation, is_frozen, scale,

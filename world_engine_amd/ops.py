@@ -49,10 +49,9 @@ _initialised = set()   # (library handle id, device index) pairs whose one-time 
 
 def init(device=None, probe: bool = False) -> None:
     """One-time set-up of a device for the library (``we_init``): kernel LDS limits, the static
-    scratch buffer's address, and a small probe launch that checks the workgroup -> XCD mapping the
-    in-kernel merge of split-context parts relies on.  Synchronises the device once.  Every wrapper
-    here does it on first use; code that captures HIP graphs without an eager warm-up call calls
-    this first (the set-up cannot run under capture)."""
+    scratch buffer's address, the compute-unit count.  Every wrapper here does it on first use;
+    code that captures HIP graphs without an eager warm-up call calls this first (the set-up's
+    runtime calls do not belong into a capture)."""
     dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
     if dev.index is None:
         dev = torch.device("cuda", torch.cuda.current_device())
@@ -78,14 +77,6 @@ def _call(dev: torch.device, fn, *args, probe: bool = False):
         return fn(*args)
     with torch.cuda.device(dev):
         return fn(*args)
-
-
-def new_workspace(n_bytes: int, dev: torch.device) -> Tensor:
-    """A split-context workspace as the library wants to find it: the arrival counters at its start
-    zero (every call leaves them zero again), the rest uninitialised."""
-    ws = torch.empty(n_bytes, dtype=torch.uint8, device=dev)
-    ws[: _capi.WE_WS_COUNTER_BYTES].zero_()
-    return ws
 
 
 def _bhtd_strides(t: Tensor, what: str):
@@ -207,22 +198,19 @@ def attn_workspace_bytes(B: int, H: int, Hkv: int, T: int, Dh: int, L: int, n_sp
 
 
 def attn_plan(B: int, H: int, Hkv: int, T: int, Dh: int, L: int, n_splits: int = 0, q_tile: int = 0,
-              compute_units: int = 0, xcd_merge: Optional[bool] = True, two_pass: bool = False) -> dict:
+              compute_units: int = 0) -> dict:
     """What the library would do with an attention call of these sizes (``we_attn_plan``; launches
-    nothing, needs no GPU when ``compute_units`` is given).  ``xcd_merge=None``: as the current
-    device's set-up found it, i.e. what a call on that device will really do."""
+    nothing, needs no GPU when ``compute_units`` is given)."""
     out = (ctypes.c_int32 * _capi.WE_PLAN_FIELDS)()
-    code = _capi.lib().we_attn_plan(B, H, Hkv, T, Dh, L, n_splits, q_tile | (_capi.WE_SPLIT_TWO_PASS if two_pass else 0),
-                                    compute_units, -1 if xcd_merge is None else int(bool(xcd_merge)), out)
+    code = _capi.lib().we_attn_plan(B, H, Hkv, T, Dh, L, n_splits, q_tile, compute_units, out)
     _capi.check(code, "we_attn_plan")
-    return {"q_tile": out[0], "n_splits": out[1], "units_whole": out[2], "merge_in_kernel": bool(out[3]),
-            "workgroups": out[4], "compute_units": out[5]}
+    return {"q_tile": out[0], "n_splits": out[1], "units_whole": out[2], "workgroups": out[3], "compute_units": out[4]}
 
 
 def attn_ring(q: Tensor, kv: Tensor, written: Tensor, t_pos: Tensor, L: int, dilation: int,
               scale: Optional[float] = None, n_splits: int = 0, q_tile: int = 0,
               out: Optional[Tensor] = None, workspace: Optional[Tensor] = None,
-              token_major_out: bool = True, clocks: Optional[Tensor] = None, two_pass: bool = False) -> Tensor:
+              token_major_out: bool = True, clocks: Optional[Tensor] = None) -> Tensor:
     """Attention of one frame's queries over the visible part of the ring buffer.
 
     Replaces ``make_block_mask`` + ``flex_attention`` (``src/model/kv_cache.py:141-144``,
@@ -230,9 +218,7 @@ def attn_ring(q: Tensor, kv: Tensor, written: Tensor, t_pos: Tensor, L: int, dil
     ``[2,B,Hkv,L+T,Dh]``, ``written`` ``[L+T]`` bool, ``t_pos`` int64 with the frame index at
     element 0.  Returns ``[B,H,T,Dh]``; with ``token_major_out`` its memory is ``[B,T,H,Dh]`` so
     that ``y.transpose(1, 2).reshape(B, T, H*Dh)`` is a view (``src/patch_model.py:139``).
-    ``workspace`` (split-context scratch, ``new_workspace``) is allocated when not given.
-    ``two_pass`` merges split-context parts with the second kernel even where the main kernel would
-    do it itself (same bits; for comparisons).
+    ``workspace`` (split-context scratch, uint8, ``attn_workspace_bytes`` long) is allocated when not given.
     ``clocks`` (int64 device tensor): the call goes through the measurement library
     (``libwe_probe.so``, ``we_attn_ring_fwd_clocked``), which also leaves, per workgroup of the main
     kernel, its duration in shader-clock cycles and in ticks of the constant 100 MHz counter.
@@ -252,12 +238,10 @@ def attn_ring(q: Tensor, kv: Tensor, written: Tensor, t_pos: Tensor, L: int, dil
         raise RuntimeError("t_pos must be a non-empty int64 tensor")
     scale = 1.0 / math.sqrt(Dh) if scale is None else float(scale)
     lib = _capi.probe_lib() if clocks is not None else _capi.lib()
-    if two_pass:
-        q_tile |= _capi.WE_SPLIT_TWO_PASS
     with torch.cuda.device(dev):      # (the size depends on the device's compute-unit count)
         ws_bytes = int(lib.we_attn_workspace_bytes(B, H, Hkv, T, Dh, L, n_splits, q_tile))
     if ws_bytes and (workspace is None or workspace.numel() * workspace.element_size() < ws_bytes):
-        workspace = new_workspace(ws_bytes, dev)
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     if out is None:
         if token_major_out:
             out = torch.empty((B, T, H, Dh), dtype=q.dtype, device=dev).transpose(1, 2)
@@ -394,7 +378,7 @@ def rope_kv_attn(q: Tensor, k: Tensor, v: Tensor, pos_ids: Mapping[str, Tensor],
     with torch.cuda.device(dev):
         ws_bytes = int(lib.we_attn_workspace_bytes(B, H, Hkv, T, Dh, L, n_splits, q_tile))
     if ws_bytes and (workspace is None or workspace.numel() * workspace.element_size() < ws_bytes):
-        workspace = new_workspace(ws_bytes, dev)
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     if q_rot is None:
         q_rot = torch.empty((B, H, T, Dh), dtype=q.dtype, device=dev)
     elif tuple(q_rot.shape) != (B, H, T, Dh) or q_rot.dtype != q.dtype or q_rot.device != dev or not q_rot.is_contiguous():
@@ -488,7 +472,7 @@ def qkv_rope_kv_attn(x: Tensor, w_qkv: Tensor, n_heads: int, n_kv_heads: int, po
         return None, q_rot, v_raw
     with torch.cuda.device(dev):
         ws_bytes = int(lib.we_attn_workspace_bytes(B, H, Hkv, T, Dh, L, n_splits, q_tile))
-    workspace = buf(("workspace", ws_bytes), lambda: new_workspace(ws_bytes, dev)) if ws_bytes else None
+    workspace = buf(("workspace", ws_bytes), lambda: torch.empty(ws_bytes, dtype=torch.uint8, device=dev)) if ws_bytes else None
     out = buf("out", lambda: torch.empty((B, T, H, Dh), dtype=x.dtype, device=dev).transpose(1, 2))
     code = _call(dev, lib.we_qkv_rope_kv_attn_fwd, *head, out.data_ptr(), _bhtd_strides(out, "out"),
                  workspace.data_ptr() if ws_bytes else None, ws_bytes,
